@@ -1,0 +1,9 @@
+"""RNN-T loss and gradient for compact-layout inputs on AMD MI355X (gfx950).
+
+`transducer_loss` keeps the entry point of CompactWarpRNNTLoss (cwarp_rnnt/__init__.py:32-73);
+the work is done by hand-written HIP kernels behind the C ABI of include/cwarp_rnnt_hip.h.
+"""
+from .loss import ForwardState, rnnt_backward, rnnt_forward, transducer_loss  # noqa: F401
+
+__version__ = "0.1.0"
+__all__ = ["transducer_loss", "rnnt_forward", "rnnt_backward", "ForwardState", "__version__"]

@@ -1,0 +1,221 @@
+// extern "C" entry points of libcwarp_rnnt_hip.so: argument validation (host only, before any HIP
+// call), workspace carving and kernel sequencing.  Mirrors the orchestration of
+// cwarp_cuda.cpp:58-136 without its host synchronisations and allocations.
+#include "cwr_device.hpp"
+#include "cwr_host.hpp"
+
+namespace cwr {
+
+static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct Layout {
+    size_t lp, alpha, beta, bnd_a, bnd_b, total;
+};
+
+static Layout layout_for(i64 N, i64 R) {
+    (void)N;
+    Layout l;
+    size_t cells = (size_t)(R > 0 ? R : 0);
+    size_t bnd = (cells >> 6) + 1;
+    size_t at = 0;
+    l.lp = at; at = align_up(at + cells * sizeof(float2));
+    l.alpha = at; at = align_up(at + cells * sizeof(double));
+    l.beta = at; at = align_up(at + cells * sizeof(double));
+    l.bnd_a = at; at = align_up(at + bnd * sizeof(double));
+    l.bnd_b = at; at = align_up(at + bnd * sizeof(double));
+    l.total = at;
+    return l;
+}
+
+size_t workspace_bytes(i64 N, i64 R) { return layout_for(N, R).total; }
+
+bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, Workspace* ws) {
+    Layout l = layout_for(N, R);
+    if (bytes < l.total) return false;
+    char* p = static_cast<char*>(base);
+    ws->lp = reinterpret_cast<float2*>(p + l.lp);
+    ws->alpha = reinterpret_cast<double*>(p + l.alpha);
+    ws->beta = reinterpret_cast<double*>(p + l.beta);
+    ws->bnd_a = reinterpret_cast<double*>(p + l.bnd_a);
+    ws->bnd_b = reinterpret_cast<double*>(p + l.bnd_b);
+    return true;
+}
+
+int workspace_section(i64 N, i64 R, int which, size_t* offset, size_t* bytes) {
+    if (!offset || !bytes) return CWR_ERR_NULL;
+    if (N < 0 || R < 0) return CWR_ERR_SHAPE;
+    Layout l = layout_for(N, R);
+    switch (which) {
+        case 0: *offset = l.lp; *bytes = (size_t)R * sizeof(float2); return CWR_OK;
+        case 1: *offset = l.alpha; *bytes = (size_t)R * sizeof(double); return CWR_OK;
+        case 2: *offset = l.beta; *bytes = (size_t)R * sizeof(double); return CWR_OK;
+    }
+    return CWR_ERR_SHAPE;
+}
+
+static size_t elem_size(int dtype) {
+    switch (dtype) {
+        case CWR_F32: return 4;
+        case CWR_F16: return 2;
+        case CWR_BF16: return 2;
+        case CWR_F64: return 8;
+    }
+    return 0;
+}
+
+static bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+// Checks shared by the three compute entry points.
+static int check_common(const void* x, bool need_x, int dtype, int64_t R, int64_t V, const int32_t* lx,
+                        const int32_t* ly, const int32_t* y, int64_t y_len, int64_t N, int32_t blank,
+                        int mode) {
+    if (dtype < CWR_F32 || dtype > CWR_F64) return CWR_ERR_DTYPE;
+    if (mode != CWR_MODE_LOGPROB && mode != CWR_MODE_FUSED) return CWR_ERR_MODE;
+    if (N < 0 || R < 0 || V < 1 || y_len < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff || V > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (R > 0 && N == 0) return CWR_ERR_SHAPE;
+    if (blank < 0 || blank >= V) return CWR_ERR_BLANK;
+    if (N > 0 && (!lx || !ly)) return CWR_ERR_NULL;
+    if (y_len > 0 && !y) return CWR_ERR_NULL;
+    if (need_x && R > 0 && !x) return CWR_ERR_NULL;
+    if (x && misaligned(x, elem_size(dtype))) return CWR_ERR_ALIGN;
+    if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(y, 4)) return CWR_ERR_ALIGN;
+    return CWR_OK;
+}
+
+static Batch make_batch(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                        const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                        int64_t max_u, const int64_t* row_off, const int64_t* lab_off, int32_t* status,
+                        void* stream) {
+    Batch b;
+    b.x = x; b.dtype = dtype; b.R = R; b.V = (int)V; b.lx = lx; b.ly = ly; b.y = y;
+    b.y_stride = y_stride; b.y_len = y_len; b.N = (int)N; b.blank = blank; b.mode = mode; b.max_u = max_u;
+    b.row_off = reinterpret_cast<const i64*>(row_off);
+    b.lab_off = reinterpret_cast<const i64*>(lab_off);
+    b.status = status;
+    b.stream = static_cast<hipStream_t>(stream);
+    return b;
+}
+
+}  // namespace cwr
+
+using namespace cwr;
+
+extern "C" {
+
+int cwr_version(void) { return 100; }
+
+const char* cwr_strerror(int status) {
+    switch (status) {
+        case CWR_OK: return "success";
+        case CWR_ERR_NULL: return "a required pointer is NULL";
+        case CWR_ERR_DTYPE: return "unsupported dtype (expected CWR_F32, CWR_F16, CWR_BF16 or CWR_F64)";
+        case CWR_ERR_MODE: return "unsupported mode (expected CWR_MODE_LOGPROB or CWR_MODE_FUSED)";
+        case CWR_ERR_SHAPE: return "negative or inconsistent sizes";
+        case CWR_ERR_BLANK: return "blank index outside [0, V)";
+        case CWR_ERR_ALIGN: return "a buffer is not aligned to its element size";
+        case CWR_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
+        case CWR_ERR_TOO_LARGE: return "a size exceeds what the kernels can index";
+    }
+    return "unknown status";
+}
+
+size_t cwr_workspace_bytes(int64_t N, int64_t R) {
+    if (N < 0 || R < 0) return 0;
+    return workspace_bytes(N, R);
+}
+
+int cwr_workspace_section(int64_t N, int64_t R, int which, size_t* offset, size_t* bytes) {
+    return workspace_section(N, R, which, offset, bytes);
+}
+
+int64_t cwr_diag_index(int64_t t, int64_t u, int64_t T, int64_t U) {
+    if (t < 0 || u < 0 || t >= T || u > U) return -1;
+    return diag_index(t, u, T, U + 1);
+}
+
+int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int64_t* row_off,
+                int64_t* lab_off, int32_t* status, void* stream) {
+    if (N < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (!row_off || !lab_off || !status || (N > 0 && (!lx || !ly))) return CWR_ERR_NULL;
+    if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(row_off, 8) || misaligned(lab_off, 8) ||
+        misaligned(status, 4))
+        return CWR_ERR_ALIGN;
+    return launch_offsets(lx, ly, N, R, reinterpret_cast<i64*>(row_off), reinterpret_cast<i64*>(lab_off),
+                          status, nullptr, static_cast<hipStream_t>(stream));
+}
+
+static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                        const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                        int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
+                        int64_t* lab_off, int32_t* status, float* lse, float* grads, float* costs,
+                        void* stream, bool with_grad) {
+    int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+    if (rc != CWR_OK) return rc;
+    if (max_u < 0) return CWR_ERR_SHAPE;
+    if (!row_off || !lab_off || !status) return CWR_ERR_NULL;
+    if (N > 0 && !costs) return CWR_ERR_NULL;
+    if (R > 0 && !workspace) return CWR_ERR_NULL;
+    if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
+    if (R > 0 && with_grad && !grads) return CWR_ERR_NULL;
+    if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
+        misaligned(grads, 8) || misaligned(costs, 4) || misaligned(workspace, 256))
+        return CWR_ERR_ALIGN;
+    Workspace ws;
+    if (!carve_workspace(workspace, workspace_bytes_, N, R, &ws)) return CWR_ERR_SHAPE;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    rc = launch_offsets(lx, ly, N, R, reinterpret_cast<i64*>(row_off), reinterpret_cast<i64*>(lab_off),
+                        status, costs, s);
+    if (rc != CWR_OK) return rc;
+    Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
+                         status, stream);
+    rc = launch_gather(b, ws, lse);
+    if (rc != CWR_OK) return rc;
+    rc = launch_lattice(b, ws, !with_grad);
+    if (rc != CWR_OK) return rc;
+    if (with_grad) return launch_fill(b, ws, grads, costs);
+    return launch_cost_from_beta(b, ws, costs);
+}
+
+int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
+                int32_t* status, float* lse, float* grads, float* costs, void* stream) {
+    return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                        workspace_bytes_, row_off, lab_off, status, lse, grads, costs, stream, true);
+}
+
+int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+             const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+             int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
+             int32_t* status, float* costs, void* stream) {
+    // the fused gather still needs somewhere to put lse; it lives in the alpha slot, unused here
+    Workspace ws;
+    float* lse = nullptr;
+    if (workspace && carve_workspace(workspace, workspace_bytes_, N, R, &ws))
+        lse = reinterpret_cast<float*>(ws.alpha);
+    return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                        workspace_bytes_, row_off, lab_off, status, lse, nullptr, costs, stream, false);
+}
+
+int cwr_backward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                 const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                 const int64_t* row_off, const int64_t* lab_off, const float* grads, const float* lse,
+                 const float* grad_costs, void* grad_x, void* stream) {
+    int rc = check_common(x, mode == CWR_MODE_FUSED, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+    if (rc != CWR_OK) return rc;
+    if (!row_off || !lab_off) return CWR_ERR_NULL;
+    if (R > 0 && (!grads || !grad_x || !grad_costs)) return CWR_ERR_NULL;
+    if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
+    if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(grads, 8) || misaligned(lse, 4) ||
+        misaligned(grad_costs, 4) || misaligned(grad_x, elem_size(dtype)))
+        return CWR_ERR_ALIGN;
+    // no status word here: the forward pass has already flagged bad labels
+    Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, 0, row_off, lab_off,
+                         nullptr, stream);
+    return launch_grad(b, grads, lse, grad_costs, grad_x);
+}
+
+}  // extern "C"

@@ -1,0 +1,243 @@
+// Device-side helpers shared by the kernels: wave64 cross-lane primitives (DPP), element packs
+// for 128-bit global accesses, and the index arithmetic of the compact and anti-diagonal layouts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/cwarp_rnnt_hip.h"
+
+namespace cwr {
+
+typedef long long i64;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+// "no path" marker of the lattice recursions.  Finite, so that marker - marker = 0 instead of NaN.
+constexpr double kNeg = -1.0e30;
+
+// ---------------------------------------------------------------------------------------------
+// wave64 cross-lane moves.  gfx9-family DPP controls.
+// ---------------------------------------------------------------------------------------------
+constexpr int DPP_QUAD_XOR1 = 0xB1;    // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;    // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_SHR = 0x110;     // + n
+constexpr int DPP_WAVE_SHL1 = 0x130;   // lane i reads lane i+1
+constexpr int DPP_WAVE_SHR1 = 0x138;   // lane i reads lane i-1
+constexpr int DPP_ROW_MIRROR = 0x140;
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_BCAST15 = 0x142;
+constexpr int DPP_ROW_BCAST31 = 0x143;
+
+// Lanes without a valid source (or masked off by ROW_MASK) return `old`.
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32(float old, float src) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src),
+                                                      CTRL, ROW_MASK, BANK_MASK, false));
+}
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ int dpp_i32(int old, int src) {
+    return __builtin_amdgcn_update_dpp(old, src, CTRL, ROW_MASK, BANK_MASK, false);
+}
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ i64 dpp_i64(i64 old, i64 src) {
+    int lo = dpp_i32<CTRL, ROW_MASK, BANK_MASK>((int)(old & 0xffffffffLL), (int)(src & 0xffffffffLL));
+    int hi = dpp_i32<CTRL, ROW_MASK, BANK_MASK>((int)(old >> 32), (int)(src >> 32));
+    return ((i64)hi << 32) | (i64)(unsigned)lo;
+}
+
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ double dpp_f64(double old, double src) {
+    int lo = dpp_i32<CTRL, ROW_MASK, BANK_MASK>(__double2loint(old), __double2loint(src));
+    int hi = dpp_i32<CTRL, ROW_MASK, BANK_MASK>(__double2hiint(old), __double2hiint(src));
+    return __hiloint2double(hi, lo);
+}
+
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+    int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
+    int hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+    return __hiloint2double(hi, lo);
+}
+
+__device__ __forceinline__ float readlane_f32(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+struct OpMax {
+    static __device__ __forceinline__ float identity() { return -INFINITY; }
+    static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
+};
+struct OpSum {
+    static __device__ __forceinline__ float identity() { return 0.0f; }
+    static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+
+// All-reduce over aligned groups of W consecutive lanes (W a power of two, 1..64): every lane of
+// a group ends up with the group's result.
+template <int W, class Op>
+__device__ __forceinline__ float group_allreduce(float v) {
+    if (W >= 2) v = Op::apply(v, dpp_f32<DPP_QUAD_XOR1>(v, v));
+    if (W >= 4) v = Op::apply(v, dpp_f32<DPP_QUAD_XOR2>(v, v));
+    if (W >= 8) v = Op::apply(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v, v));
+    if (W >= 16) v = Op::apply(v, dpp_f32<DPP_ROW_MIRROR>(v, v));
+    if (W == 32) v = Op::apply(v, __shfl_xor(v, 16));
+    if (W == 64) {
+        // rows 1,3 += row 0,2 ; rows 2,3 += lane 31 ; lane 63 then holds the total
+        v = Op::apply(v, dpp_f32<DPP_ROW_BCAST15, 0xA>(Op::identity(), v));
+        v = Op::apply(v, dpp_f32<DPP_ROW_BCAST31, 0xC>(Op::identity(), v));
+        v = readlane_f32(v, 63);
+    }
+    return v;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ i64 wave_inclusive_scan(i64 v) {
+    v += dpp_i64<DPP_ROW_SHR + 1>(0, v);
+    v += dpp_i64<DPP_ROW_SHR + 2>(0, v);
+    v += dpp_i64<DPP_ROW_SHR + 4>(0, v);
+    v += dpp_i64<DPP_ROW_SHR + 8>(0, v);
+    v += dpp_i64<DPP_ROW_BCAST15, 0xA>(0, v);
+    v += dpp_i64<DPP_ROW_BCAST31, 0xC>(0, v);
+    return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// log(exp(a)+exp(b)) = max + log1p(exp(-|a-b|)), the form of cwarp_cuda_rnnt_kernel.cu:22-29.
+// The running values are kept in fp64 (a lattice of ~2000 steps reaches magnitudes of several
+// thousand, where an fp32 ulp is already 2e-4); the correction term, at most ln 2, is evaluated
+// on the fp32 exp2/log2 units from the fp32-rounded difference.
+__device__ __forceinline__ double log_sum_exp(double a, double b) {
+    double mx = fmax(a, b);
+    float d = -fabsf((float)(a - b));
+    float e = fast_exp2(d * kLog2e);
+    return mx + (double)(fast_log2(1.0f + e) * kLn2);
+}
+
+// ---------------------------------------------------------------------------------------------
+// element packs: VEC consecutive elements moved with one 16-byte access, computed on as fp32
+// ---------------------------------------------------------------------------------------------
+struct bf16_t { uint16_t v; };
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+};
+template <> struct Elem<__half> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ float to_f32(__half v) { return __half2float(v); }
+    static __device__ __forceinline__ __half from_f32(float v) { return __float2half_rn(v); }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.v << 16); }
+    static __device__ __forceinline__ bf16_t from_f32(float f) {
+        uint32_t u = __float_as_uint(f);
+        bf16_t r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) { r.v = (uint16_t)((u >> 16) | 0x40); return r; }  // NaN
+        u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+        r.v = (uint16_t)(u >> 16);
+        return r;
+    }
+};
+template <> struct Elem<double> {
+    static constexpr int VEC = 2;
+    static __device__ __forceinline__ float to_f32(double v) { return (float)v; }
+    static __device__ __forceinline__ double from_f32(float v) { return (double)v; }
+};
+
+template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PackT { T e[VEC]; };
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_pack(const T* __restrict__ p, float (&out)[VEC]) {
+    PackT<T, VEC> raw = *reinterpret_cast<const PackT<T, VEC>*>(p);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) out[i] = Elem<T>::to_f32(raw.e[i]);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void store_pack(T* __restrict__ p, const float (&in)[VEC]) {
+    PackT<T, VEC> raw;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) raw.e[i] = Elem<T>::from_f32(in[i]);
+    *reinterpret_cast<PackT<T, VEC>*>(p) = raw;
+}
+
+// ---------------------------------------------------------------------------------------------
+// layouts
+// ---------------------------------------------------------------------------------------------
+// Anti-diagonal order of a T x Up lattice: diagonals k = t+u ascending, inside a diagonal u
+// ascending.  diag_start(k) = number of cells on diagonals < k.
+__host__ __device__ __forceinline__ i64 diag_start(i64 k, i64 T, i64 Up) {
+    i64 m = T < Up ? T : Up;
+    i64 M = T < Up ? Up : T;
+    if (k <= m) return k * (k + 1) / 2;
+    if (k <= M) return m * (m + 1) / 2 + (k - m) * m;
+    i64 j = k - M;
+    return m * (m + 1) / 2 + (M - m) * m + j * (m - 1) - j * (j - 1) / 2;
+}
+__host__ __device__ __forceinline__ i64 diag_count(i64 k, i64 T, i64 Up) {
+    i64 hi = k < Up - 1 ? k : Up - 1;
+    i64 lo = k - (T - 1) > 0 ? k - (T - 1) : 0;
+    return hi - lo + 1;
+}
+__host__ __device__ __forceinline__ i64 diag_index(i64 t, i64 u, i64 T, i64 Up) {
+    i64 k = t + u;
+    i64 lo = k - (T - 1) > 0 ? k - (T - 1) : 0;
+    return diag_start(k, T, Up) + (u - lo);
+}
+
+// Which sequence owns compact row r, and where in its lattice the row sits.
+struct RowInfo {
+    int n;    // -1: the row belongs to no usable sequence
+    int t, u;
+    int T, U;
+    i64 off;  // row_off[n]
+};
+
+__device__ __forceinline__ RowInfo decode_row(i64 r, i64 R, const i64* __restrict__ row_off,
+                                              const int* __restrict__ lx, const int* __restrict__ ly,
+                                              int N) {
+    RowInfo ri;
+    ri.n = -1; ri.t = 0; ri.u = 0; ri.T = 0; ri.U = 0; ri.off = 0;
+    if (N <= 0) return ri;
+    int lo = 0, hi = N - 1;
+    while (lo < hi) {  // last n with row_off[n] <= r (skips empty sequences)
+        int mid = (lo + hi + 1) >> 1;
+        if (row_off[mid] <= r) lo = mid; else hi = mid - 1;
+    }
+    i64 off = row_off[lo];
+    int T = lx[lo], U = ly[lo];
+    if (T <= 0 || U < 0) return ri;
+    i64 cells = (i64)T * (i64)(U + 1);
+    i64 rem = r - off;
+    if (rem < 0 || rem >= cells || off + cells > R) return ri;
+    ri.n = lo; ri.T = T; ri.U = U; ri.off = off;
+    if (cells < 0x7fffffffLL) {
+        unsigned q = (unsigned)rem / (unsigned)(U + 1);
+        ri.t = (int)q;
+        ri.u = (int)((unsigned)rem - q * (unsigned)(U + 1));
+    } else {
+        ri.t = (int)(rem / (U + 1));
+        ri.u = (int)(rem - (i64)ri.t * (U + 1));
+    }
+    return ri;
+}
+
+__device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restrict__ y, i64 y_stride,
+                                           i64 y_len, const i64* __restrict__ lab_off, int V,
+                                           int* status) {
+    if (ri.n < 0 || ri.u >= ri.U) return -1;
+    i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : lab_off[ri.n]) + ri.u;
+    int lab = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
+    if (lab < 0 || lab >= V) {
+        if (status) atomicOr(status, CWR_FLAG_BAD_LABEL);
+        return -1;
+    }
+    return lab;
+}
+
+}  // namespace cwr

@@ -1,0 +1,62 @@
+// Host-side declarations shared by the translation units of libcwarp_rnnt_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/cwarp_rnnt_hip.h"
+
+namespace cwr {
+
+typedef long long i64;
+
+// One batch as the kernels see it.
+struct Batch {
+    const void* x;
+    int dtype;
+    i64 R;
+    int V;
+    const int* lx;
+    const int* ly;
+    const int* y;
+    i64 y_stride;
+    i64 y_len;
+    int N;
+    int blank;
+    int mode;
+    i64 max_u;
+    const i64* row_off;
+    const i64* lab_off;
+    int* status;
+    hipStream_t stream;
+};
+
+// Scratch carved out of the caller's workspace.  Cells of a sequence are stored in anti-diagonal
+// order (see diag_index).
+struct Workspace {
+    float2* lp;     // R    gathered (blank, label) log-probabilities
+    double* alpha;  // R
+    double* beta;   // R
+    double* bnd_a;  // R/64+1  alpha values handed from one 64-label strip to the next
+    double* bnd_b;  // R/64+1  same for beta
+};
+
+size_t workspace_bytes(i64 N, i64 R);
+bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, Workspace* ws);
+int workspace_section(i64 N, i64 R, int which, size_t* offset, size_t* bytes);
+
+int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64* row_off, i64* lab_off,
+                   int* status, float* costs_or_null, hipStream_t stream);
+int launch_gather(const Batch& b, const Workspace& ws, float* lse);
+int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
+int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs);
+int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs);
+int launch_grad(const Batch& b, const float* grads, const float* lse, const float* grad_costs,
+                void* grad_x);
+
+inline int check_launch() {
+    return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;
+}
+
+}  // namespace cwr

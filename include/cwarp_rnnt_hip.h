@@ -1,0 +1,143 @@
+/*
+ * cwarp_rnnt_hip.h -- C ABI of libcwarp_rnnt_hip.so: RNN-T loss and gradient for compact-layout
+ * inputs on AMD MI355X (gfx950).
+ *
+ * The three compute entry points replace the three functions the reference exports through
+ * pybind11 (CompactWarpRNNTLoss, cwarp_cuda.cpp:138-153):
+ *
+ *     _cwarp_rnnt_forward   (cwarp_cuda.cpp:84-108)   ->  cwr_forward
+ *     _cwarp_rnnt_loss      (cwarp_cuda.cpp:58-82)    ->  cwr_loss
+ *     _cwarp_rnnt_backward  (cwarp_cuda.cpp:110-136)  ->  cwr_backward
+ *
+ * plus cwr_offsets for the row-offset computation the reference repeats inline in each of them
+ * (cwarp_cuda.cpp:72-77, 98-103, 124-129).
+ *
+ * Conventions
+ *   - Every pointer named below is a DEVICE pointer unless stated otherwise.  The library never
+ *     allocates, frees or synchronises; all kernels are enqueued on `stream` (a hipStream_t
+ *     passed as void*; NULL = the default stream).
+ *   - Every function returns a cwr_status (0 = success).  Argument validation happens on the
+ *     host before any HIP call, so invalid calls can be exercised without a GPU.
+ *   - Data-dependent problems (lengths that do not add up to R, labels outside [0,V), ...) cannot
+ *     be seen by the host without a synchronisation; kernels guard every access, never touch
+ *     memory outside the given buffers, and record CWR_FLAG_* bits in status[0].
+ *   - Compact layout: x has R = sum_n lx[n]*(ly[n]+1) rows of V entries; the row of sequence n,
+ *     frame t, label position u is row_off[n] + t*(ly[n]+1) + u
+ *     (cwarp_cuda_gather_kernel.cu:36, test/test.py:44-46).
+ *   - Labels: y_stride >= 0 -> padded 2-D labels, label u of sequence n is y[n*y_stride + u]
+ *     (the reference layout, cwarp_rnnt/__init__.py:45-49);
+ *     y_stride < 0 -> concatenated 1-D labels, label u of sequence n is y[lab_off[n] + u].
+ *     y_len is the number of int32 entries behind y; reads beyond it are refused and flagged.
+ */
+#ifndef CWARP_RNNT_HIP_H
+#define CWARP_RNNT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of x and of the gradient w.r.t. x (all arithmetic is done in fp32) */
+enum cwr_dtype { CWR_F32 = 0, CWR_F16 = 1, CWR_BF16 = 2, CWR_F64 = 3 };
+
+/* CWR_MODE_LOGPROB: x holds log-probabilities; the gradient is non-zero only in the blank and
+ *                   label columns (exactly what the reference computes).
+ * CWR_MODE_FUSED:   x holds raw logits; log-softmax over V is fused into the gather pass and the
+ *                   gradient w.r.t. the logits is dense. */
+enum cwr_mode { CWR_MODE_LOGPROB = 0, CWR_MODE_FUSED = 1 };
+
+enum cwr_status {
+    CWR_OK = 0,
+    CWR_ERR_NULL = 1,      /* a required pointer is NULL */
+    CWR_ERR_DTYPE = 2,     /* dtype is not a cwr_dtype */
+    CWR_ERR_MODE = 3,      /* mode is not a cwr_mode */
+    CWR_ERR_SHAPE = 4,     /* negative or inconsistent N, R, V, max_u */
+    CWR_ERR_BLANK = 5,     /* blank outside [0, V) (cwarp_rnnt/__init__.py:50) */
+    CWR_ERR_ALIGN = 6,     /* a buffer is not aligned to its element size */
+    CWR_ERR_LAUNCH = 7,    /* the HIP runtime refused a launch */
+    CWR_ERR_TOO_LARGE = 8  /* a size exceeds what the kernels index */
+};
+
+/* bits of status[0], written by the kernels */
+enum cwr_flag {
+    CWR_FLAG_ROWS_MISMATCH = 1, /* sum lx*(ly+1) != R */
+    CWR_FLAG_BAD_LENGTH = 2,    /* some lx <= 0 or ly < 0 (that sequence is skipped, cost = NaN) */
+    CWR_FLAG_BAD_LABEL = 4,     /* a label outside [0, V) was met (treated as "no label") */
+    CWR_FLAG_FB_MISMATCH = 8,   /* forward and backward likelihood differ by > 0.1 % for some
+                                   sequence; the cost is their mean, as in the reference
+                                   (cwarp_cuda_rnnt_kernel.cu:356-364, which prints instead) */
+    CWR_FLAG_U_TOO_LARGE = 16   /* some ly exceeds the max_u given to the call */
+};
+
+int cwr_version(void);
+const char* cwr_strerror(int status);
+
+/* Bytes of scratch cwr_forward / cwr_loss need for a batch of N sequences and R rows.  The
+ * scratch holds the gathered log-probabilities, alpha and beta (all O(R)); nothing in it is
+ * needed by cwr_backward. */
+size_t cwr_workspace_bytes(int64_t N, int64_t R);
+
+/* Location of alpha / beta inside the workspace after cwr_forward, for analysis tools (the
+ * reference returns both, cwarp_cuda_rnnt_kernel.cu:383-384).  which: 0 = gathered log-probs
+ * (float2 per cell), 1 = alpha, 2 = beta (float per cell).  Cells are stored per sequence in
+ * anti-diagonal order: cell (t,u) of sequence n lives at row_off[n] + cwr_diag_index(t,u,T,U). */
+int cwr_workspace_section(int64_t N, int64_t R, int which, size_t* offset, size_t* bytes);
+int64_t cwr_diag_index(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
+
+/* Row and label offsets by a device prefix scan.
+ *   row_off[n] = sum_{j<n} lx[j]*(ly[j]+1), n = 0..N   (N+1 entries, int64)
+ *   lab_off[n] = sum_{j<n} ly[j],           n = 0..N   (N+1 entries, int64)
+ * Replaces cwarp_cuda.cpp:72-77 (which keeps the first N entries as int32).
+ * status: 4 x int32, zeroed then flagged.  R < 0 skips the row-count check. */
+int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R,
+                int64_t* row_off, int64_t* lab_off, int32_t* status, void* stream);
+
+/* Loss with the state the backward pass needs.  Replaces _cwarp_rnnt_forward
+ * (cwarp_cuda.cpp:84-108 -> gather_cuda_forward + cwarp_cuda_costs_with_grad).
+ *   x        (R,V) of `dtype`, contiguous
+ *   lx, ly   (N,) int32 frame / label counts;  y, y_stride: labels (see above)
+ *   max_u    an upper bound of max(ly) known to the host (e.g. the padded label width)
+ * outputs
+ *   row_off, lab_off (N+1) int64;  status 4 x int32
+ *   lse      (R,) fp32 log-sum-exp of each row            [CWR_MODE_FUSED only, else may be NULL]
+ *   grads    (R,2) fp32 d cost / d(blank log-prob, label log-prob) per row, as the reference's
+ *            `grads` (cwarp_cuda_rnnt_kernel.cu:275-332)
+ *   costs    (N,) fp32 -log P(y|x)  (cwarp_cuda_rnnt_kernel.cu:334-367) */
+int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
+                const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                int64_t N, int32_t blank, int mode, int64_t max_u,
+                void* workspace, size_t workspace_bytes,
+                int64_t* row_off, int64_t* lab_off, int32_t* status,
+                float* lse, float* grads, float* costs, void* stream);
+
+/* Loss only (no gradient state).  Replaces _cwarp_rnnt_loss (cwarp_cuda.cpp:58-82 ->
+ * gather_cuda_forward + cwarp_cuda_cal_costs): beta recursion only, costs = -beta[0][0]. */
+int cwr_loss(const void* x, int dtype, int64_t R, int64_t V,
+             const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+             int64_t N, int32_t blank, int mode, int64_t max_u,
+             void* workspace, size_t workspace_bytes,
+             int64_t* row_off, int64_t* lab_off, int32_t* status,
+             float* costs, void* stream);
+
+/* Gradient w.r.t. x.  Replaces _cwarp_rnnt_backward (cwarp_cuda.cpp:110-136 ->
+ * cwarp_cuda_backward_ + zeros(R,V) + gather_cuda_backward_) in one streaming pass that does
+ * not modify `grads`.
+ *   CWR_MODE_LOGPROB: grad_x[r,:] = 0 except [blank] = grads[r,0]*g and [label] = grads[r,1]*g
+ *                     (label written after blank, cwarp_cuda_gather_kernel.cu:70-73); x unused.
+ *   CWR_MODE_FUSED:   grad_x[r,v] = g*(softmax(x_r)[v]*gamma_r + grads[r,0][v==blank]
+ *                     + grads[r,1][v==label]),  gamma_r = -(grads[r,0]+grads[r,1]).
+ * with g = grad_costs[n] of the row's sequence (cwarp_cuda_rnnt_kernel.cu:518-519).
+ *   grad_x   (R,V) of `dtype`, fully written. */
+int cwr_backward(const void* x, int dtype, int64_t R, int64_t V,
+                 const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                 int64_t N, int32_t blank, int mode,
+                 const int64_t* row_off, const int64_t* lab_off,
+                 const float* grads, const float* lse, const float* grad_costs,
+                 void* grad_x, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CWARP_RNNT_HIP_H */

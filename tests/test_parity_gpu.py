@@ -1,0 +1,256 @@
+"""GPU parity: the HIP path (through the C ABI) against the float64 oracle on the same seeded
+inputs.  Gates: loss <= 1e-5 relative, gradients <= 1e-4 absolute (fp32), offsets and flags exact.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import rnnt_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+GRAD_ATOL = 1e-4
+
+TORCH_DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "f64": torch.float64}
+
+
+def _pkg():
+    import compactwarprnntloss_amd as pkg
+    return pkg
+
+
+def make_batch(lx, ly, V, seed, sigma=1.0, dtype="f32", blank=0, normalised=False):
+    rng = np.random.default_rng(seed)
+    lx = np.asarray(lx, dtype=np.int32)
+    ly = np.asarray(ly, dtype=np.int32)
+    N = len(lx)
+    R = int(orc.row_offsets_i64(lx, ly)[-1])
+    x = (rng.standard_normal((R, V)) * sigma).astype(np.float32)
+    if normalised:
+        x = orc.log_softmax(x).astype(np.float32)
+    Umax = int(ly.max()) if N else 0
+    yp = np.zeros((N, Umax), dtype=np.int32)
+    for n in range(N):
+        lab = rng.integers(0, V - 1, int(ly[n])).astype(np.int32)
+        lab[lab >= blank] += 1  # any symbol but the blank
+        yp[n, : ly[n]] = lab
+    yc = np.concatenate([yp[n, : ly[n]] for n in range(N)]) if N else np.zeros(0, np.int32)
+    tdt = TORCH_DT[dtype]
+    xt = torch.from_numpy(x).to(tdt)
+    x_ref = xt.to(torch.float64).numpy()  # what the device actually sees, exactly
+    return dict(lx=lx, ly=ly, yp=yp, yc=yc, x=xt, x_ref=x_ref, V=V, R=R, N=N, blank=blank)
+
+
+def run_device(b, fused, labels="2d", grad_out=None, with_grad=True, max_u=None):
+    pkg = _pkg()
+    dev = torch.device("cuda:0")
+    xs = b["x"].to(dev)
+    lx = torch.from_numpy(b["lx"]).to(dev)
+    ly = torch.from_numpy(b["ly"]).to(dev)
+    ys = torch.from_numpy(b["yp"] if labels == "2d" else b["yc"]).to(dev)
+    costs, st = pkg.rnnt_forward(xs, lx, ys, ly, b["blank"], fused, max_u=max_u, with_grad=with_grad)
+    out = dict(costs=costs.cpu().numpy().astype(np.float64), flags=int(st.status[0].item()),
+               row_off=st.row_off.cpu().numpy(), lab_off=st.lab_off.cpu().numpy())
+    if with_grad:
+        out["G"] = st.grads.cpu().numpy().astype(np.float64)
+        if fused:
+            out["lse"] = st.lse.cpu().numpy().astype(np.float64)
+        go = np.ones(b["N"]) if grad_out is None else grad_out
+        g = pkg.rnnt_backward(xs, lx, ys, ly, b["blank"], st, torch.from_numpy(go).to(dev))
+        out["grad"] = g.to(torch.float64).cpu().numpy()
+    torch.cuda.synchronize()
+    return out
+
+
+def check_case(b, fused, labels="2d", dtype="f32", seed=0, with_weights=True):
+    rng = np.random.default_rng(seed + 99)
+    go = rng.uniform(-1.5, 1.5, b["N"]) if with_weights else None
+    dev = run_device(b, fused, labels, go)
+    y = b["yp"] if labels == "2d" else b["yc"]
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], y, b["ly"], b["blank"], "fused" if fused else "logprob",
+                            grad_out=go)
+    assert dev["flags"] == 0
+    assert np.array_equal(dev["row_off"], ref["row_off"])
+    assert np.array_equal(dev["lab_off"], orc.label_offsets_i64(b["ly"]))
+    np.testing.assert_allclose(dev["costs"], ref["costs"], rtol=LOSS_RTOL, atol=1e-6)
+    np.testing.assert_allclose(dev["G"], ref["G"], rtol=0, atol=GRAD_ATOL)
+    if fused:
+        np.testing.assert_allclose(dev["lse"], ref["lse"], rtol=1e-6, atol=1e-5)
+    if dtype == "f32" or dtype == "f64":
+        np.testing.assert_allclose(dev["grad"], ref["grad"], rtol=0, atol=GRAD_ATOL)
+    else:
+        rel = 1e-3 if dtype == "f16" else 8e-3  # one rounding to the storage type
+        np.testing.assert_allclose(dev["grad"], ref["grad"], rtol=rel, atol=GRAD_ATOL)
+    return dev, ref
+
+
+# ----------------------------------------------------------------------------- offsets
+def test_offsets_exact_and_flags():
+    from compactwarprnntloss_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+    for N in [1, 2, 63, 64, 65, 200, 1000]:
+        lx = rng.integers(1, 400, N).astype(np.int32)
+        ly = rng.integers(0, 120, N).astype(np.int32)
+        lxd, lyd = torch.from_numpy(lx).to(dev), torch.from_numpy(ly).to(dev)
+        ro = torch.empty(N + 1, dtype=torch.int64, device=dev)
+        lo = torch.empty(N + 1, dtype=torch.int64, device=dev)
+        st = torch.empty(4, dtype=torch.int32, device=dev)
+        R = int(orc.row_offsets_i64(lx, ly)[-1])
+        rc = lib.cwr_offsets(lxd.data_ptr(), lyd.data_ptr(), N, R, ro.data_ptr(), lo.data_ptr(),
+                             st.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        assert np.array_equal(ro.cpu().numpy(), orc.row_offsets_i64(lx, ly))
+        assert np.array_equal(lo.cpu().numpy(), orc.label_offsets_i64(ly))
+        # the reference keeps the first N entries as int32
+        assert np.array_equal(ro.cpu().numpy()[:N].astype(np.int32), orc.row_offsets(lx, ly))
+        assert st.cpu().numpy().tolist() == [0, 0, 0, 0]
+        rc = lib.cwr_offsets(lxd.data_ptr(), lyd.data_ptr(), N, R + 1, ro.data_ptr(), lo.data_ptr(),
+                             st.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0 and int(st[0].item()) == _lib.FLAG_ROWS_MISMATCH
+
+
+# ----------------------------------------------------------------------------- small shapes
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("labels", ["2d", "1d"])
+def test_config1_tiny(fused, labels):
+    cfg = orc.make_config(1)
+    b = make_batch(cfg["lx"], cfg["ly"], cfg["V"], seed=1, sigma=1.0, normalised=not fused)
+    check_case(b, fused, labels)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("T,U", [(1, 0), (1, 1), (1, 7), (5, 0), (2, 1), (9, 4), (4, 9), (1, 64), (70, 62),
+                                 (70, 63), (70, 64), (33, 127), (40, 128), (20, 200), (3, 300), (300, 3)])
+def test_edge_shapes_single_sequence(fused, T, U):
+    b = make_batch([T], [U], 16, seed=T * 1000 + U, normalised=not fused)
+    check_case(b, fused)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_ragged_mix_with_empty_label_and_single_frame(fused):
+    lx = [7, 1, 30, 2, 65, 1, 12, 90]
+    ly = [3, 5, 0, 2, 70, 0, 12, 1]
+    b = make_batch(lx, ly, 40, seed=5, normalised=not fused)
+    check_case(b, fused, "2d")
+    check_case(b, fused, "1d")
+
+
+@pytest.mark.parametrize("V", [3, 5, 32, 33, 64, 100, 128, 256, 500, 512, 1000, 1024, 2048, 4096, 4100])
+def test_vocabulary_sizes_fused(V):
+    b = make_batch([6, 3, 9], [2, 4, 1], V, seed=V, sigma=2.0)
+    check_case(b, True)
+
+
+@pytest.mark.parametrize("V", [3, 32, 33, 128, 1024, 1000])
+def test_vocabulary_sizes_logprob(V):
+    b = make_batch([6, 3, 9], [2, 4, 1], V, seed=V, normalised=True)
+    check_case(b, False)
+
+
+@pytest.mark.parametrize("blank", [0, 5, 15])
+@pytest.mark.parametrize("fused", [False, True])
+def test_blank_positions(blank, fused):
+    b = make_batch([6, 3, 9, 11], [2, 4, 1, 6], 16, seed=blank, blank=blank, normalised=not fused)
+    check_case(b, fused)
+
+
+@pytest.mark.parametrize("dtype,V", [("f16", 64), ("f16", 4096), ("bf16", 256), ("f64", 32), ("f64", 1024)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_storage_types(dtype, V, fused):
+    b = make_batch([12, 5, 20], [4, 7, 2], V, seed=V, dtype=dtype, normalised=not fused)
+    check_case(b, fused, dtype=dtype)
+
+
+def test_nograd_cost_equals_grad_cost():
+    b = make_batch([30, 11, 64, 5], [10, 11, 70, 0], 48, seed=3)
+    for fused in (False, True):
+        a = run_device(b, fused)
+        c = run_device(b, fused, with_grad=False)
+        np.testing.assert_allclose(a["costs"], c["costs"], rtol=1e-6)
+
+
+def test_label_equal_to_blank_logprob_follows_reference_overwrite():
+    b = make_batch([4, 3], [2, 2], 8, seed=8, normalised=True)
+    b["yp"][0, 0] = 0
+    b["yc"][0] = 0
+    check_case(b, False)
+    check_case(b, True)
+
+
+# ----------------------------------------------------------------------------- benchmark shapes
+@pytest.mark.parametrize("idx,scale", [(2, 0.25), (4, 0.3), (5, 0.15)])
+@pytest.mark.parametrize("fused", [False, True])
+def test_benchmark_configs_reduced(idx, scale, fused):
+    cfg = orc.make_config(idx, scale=scale)
+    b = make_batch(cfg["lx"], cfg["ly"], cfg["V"], seed=idx, sigma=cfg["sigma"], normalised=not fused)
+    check_case(b, fused, "1d")
+
+
+def test_config3_reduced_fp16():
+    cfg = orc.make_config(3, scale=0.15)
+    b = make_batch(cfg["lx"], cfg["ly"], cfg["V"], seed=3, sigma=1.0, dtype="f16")
+    check_case(b, True, "2d", dtype="f16")
+
+
+# ----------------------------------------------------------------------------- entry point
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none", None])
+@pytest.mark.parametrize("fused", [False, True])
+def test_transducer_loss_autograd(reduction, fused):
+    import cwarp_rnnt
+    b = make_batch([9, 4, 15], [3, 4, 0], 24, seed=21, normalised=not fused)
+    dev = torch.device("cuda:0")
+    x = b["x"].to(dev).requires_grad_(True)
+    lx, ly = torch.from_numpy(b["lx"]).to(dev), torch.from_numpy(b["ly"]).to(dev)
+    y = torch.from_numpy(b["yp"]).to(dev)
+    loss = cwarp_rnnt.transducer_loss(x, lx, y, ly, 0, reduction, fused_log_softmax=fused, validate=True)
+    w = np.array([1.0, -2.0, 0.5])
+    if reduction in ("none", None):
+        assert loss.shape == (3,)
+        (loss * torch.from_numpy(w).to(dev, torch.float32)).sum().backward()
+        go = w
+    else:
+        assert loss.dim() == 0
+        loss.backward()
+        go = np.full(3, 1.0 / 3 if reduction == "mean" else 1.0)
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "fused" if fused else "logprob", grad_out=go)
+    want = orc.reduce_costs(ref["costs"], reduction)
+    np.testing.assert_allclose(loss.detach().cpu().numpy(), want, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), ref["grad"], atol=GRAD_ATOL)
+    # no-grad path
+    with torch.no_grad():
+        l2 = cwarp_rnnt.transducer_loss(x.detach(), lx, y, ly, 0, reduction, fused_log_softmax=fused)
+    np.testing.assert_allclose(l2.cpu().numpy(), want, rtol=LOSS_RTOL)
+
+
+def test_data_dependent_problems_are_flagged_not_faulted():
+    from compactwarprnntloss_amd import _lib
+    b = make_batch([5, 6], [2, 3], 12, seed=2)
+    # a label outside [0,V)
+    b2 = dict(b)
+    b2["yp"] = b["yp"].copy()
+    b2["yp"][1, 1] = 99
+    out = run_device(b2, True)
+    assert out["flags"] & _lib.FLAG_BAD_LABEL
+    # lengths that claim more rows than x has
+    b3 = dict(b)
+    b3["lx"] = np.array([5, 60], dtype=np.int32)
+    out = run_device(b3, True)
+    assert out["flags"] & _lib.FLAG_ROWS_MISMATCH
+    assert np.isnan(out["costs"][1]) and np.isfinite(out["costs"][0])
+    # a non-positive frame count
+    b4 = dict(b)
+    b4["lx"] = np.array([0, 6], dtype=np.int32)
+    out = run_device(b4, True)
+    assert out["flags"] & _lib.FLAG_BAD_LENGTH
+    assert np.isnan(out["costs"][0])
+    import cwarp_rnnt
+    dev = torch.device("cuda:0")
+    with pytest.raises(RuntimeError):
+        cwarp_rnnt.transducer_loss(b2["x"].to(dev), torch.from_numpy(b2["lx"]).to(dev),
+                                   torch.from_numpy(b2["yp"]).to(dev), torch.from_numpy(b2["ly"]).to(dev),
+                                   fused_log_softmax=True, validate=True)
