@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the compact RNN-T loss + gradient hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2] [--no-cpu]
+
+A step is one forward + backward of `cwarp_rnnt.transducer_loss(..., fused_log_softmax=True)` on
+one synthetic batch that is already resident in HBM.  Prints ONE JSON line.
+
+  value      algorithmic HBM bytes per step / wall time per step, in GB/s, where
+             algorithmic bytes = R*V*(2*s_x + s_g): read the logits in the forward pass, read
+             them again in the backward pass, write the gradient (R = sum T_i*(U_i+1)).
+  roofline   the gradient kernel (the dominant one: 2/3 of the bytes) timed on its own with
+             HIP events on the stream it is launched on, against the 8 TB/s HBM peak.
+  cpu_baseline  the float64 NumPy oracle timed on this host on a bounded sample of the same
+             batch; its outputs double as the parity check of the run.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+WORKLOADS = {
+    1: "c1 tiny: N=4 T~U[8,32] U~U[2,10] V=32 fp32",
+    2: "c2 BPE ASR: N=32 T~U[100,250] U~U[20,80] V=1024 fp32 logits N(0,2), blank=0, mean reduction",
+    3: "c3 large vocab: N=16 T~U[150,300] U~U[40,120] V=4096 fp16 logits N(0,1)",
+    4: "c4 ragged: N=64 T~logN(120,0.6) U~logN(30,0.7) incl. U=0 and T=1, V=512 fp32",
+    5: "c5 long-form chars: N=4 T~U[1000,1500] U~U[200,400] V=128 fp32 logits N(0,1.5)",
+}
+
+
+def measured_traffic(kernel: str, config: int):
+    """HBM bytes per launch of `kernel`, from the committed rocprofv3 counter summary, or None."""
+    path = os.path.join(ROOT, "profiles", f"traffic_c{config}.json.txt")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel)
+    except (OSError, ValueError):
+        return None
+
+
+def cpu_baseline(cfg, x_cpu, budget_s, dev_out):
+    """Time the NumPy oracle on the first sequences of the batch (at least one, then as many as fit
+    the budget) and compare the device results on those sequences."""
+    from oracle import rnnt_oracle as orc
+    off = orc.row_offsets_i64(cfg["lx"], cfg["ly"])
+    esize = x_cpu.element_size()
+    t_used, n_done, bytes_done = 0.0, 0, 0
+    loss_rel, grad_abs = 0.0, 0.0
+    N = cfg["N"]
+    while n_done < N:
+        n = n_done
+        xs = x_cpu[off[n]:off[n + 1]].to(dtype=__import__("torch").float64).numpy()
+        lab = cfg["y_padded"][n:n + 1]
+        t0 = time.perf_counter()
+        ref = orc.loss_and_grad(xs, cfg["lx"][n:n + 1], lab, cfg["ly"][n:n + 1], 0, "fused",
+                                grad_out=np.array([1.0 / N]))
+        dt = time.perf_counter() - t0
+        t_used += dt
+        n_done += 1
+        bytes_done += xs.shape[0] * cfg["V"] * 3 * esize
+        loss_rel = max(loss_rel, abs(dev_out["costs"][n] - ref["costs"][0]) / abs(ref["costs"][0]))
+        grad_abs = max(grad_abs, float(np.abs(dev_out["grad"](off[n], off[n + 1]) - ref["grad"]).max()))
+        if t_used + dt > budget_s:
+            break
+    return dict(value=bytes_done / t_used / 1e9, unit="GB/s", cores=1, kind="port",
+                sample=f"float64 NumPy oracle, first {n_done} of {N} sequences of the same batch, "
+                       f"{t_used:.1f} s",
+                ), dict(loss_rel_err=loss_rel, grad_abs_err=grad_abs, sequences_checked=n_done)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=2, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU work for the baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path is measured on ONE GPU (every sequence is independent, so a "
+                 "data-parallel trainer gives each GPU its own batch); run with --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    import compactwarprnntloss_amd as pkg
+    import cwarp_rnnt
+    from oracle import rnnt_oracle as orc
+
+    dev = torch.device("cuda:0")
+    cfg = orc.make_config(args.config)
+    tdt = torch.float16 if cfg["dtype"] == "f16" else torch.float32
+    g = torch.Generator(device="cpu").manual_seed(1000 + args.config)
+    # generated on the host in fp32, rounded once to the storage type, then made resident
+    x_cpu = (torch.randn((cfg["R"], cfg["V"]), generator=g, dtype=torch.float32) * cfg["sigma"]).to(tdt)
+    x = x_cpu.to(dev).requires_grad_(True)
+    lx = torch.from_numpy(cfg["lx"]).to(dev)
+    ly = torch.from_numpy(cfg["ly"]).to(dev)
+    y = torch.from_numpy(cfg["y_padded"]).to(dev)
+    R, V, N = cfg["R"], cfg["V"], cfg["N"]
+    esize = x.element_size()
+    bytes_step = R * V * 3 * esize
+
+    def step():
+        x.grad = None
+        loss = cwarp_rnnt.transducer_loss(x, lx, y, ly, 0, "mean", gather=True, fused_log_softmax=True)
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # per-call timing with events on the stream the kernels run on (torch's current stream)
+    xd = x.detach()
+    costs, st = pkg.rnnt_forward(xd, lx, y, ly, 0, True)
+    go = torch.full((N,), 1.0 / N, device=dev)
+    out = torch.empty_like(xd)
+    iters = max(10, args.steps)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    bwd_ms = timed(lambda: pkg.rnnt_backward(xd, lx, y, ly, 0, st, go, out=out))
+    fwd_ms = timed(lambda: pkg.rnnt_forward(xd, lx, y, ly, 0, True))
+    nograd_ms = timed(lambda: pkg.rnnt_forward(xd, lx, y, ly, 0, True, with_grad=False))
+
+    grad_bytes = R * V * 2 * esize
+    achieved = grad_bytes / (bwd_ms * 1e-3) / 1e9
+    result = {
+        "metric": "fwd+bwd algorithmic HBM GB/s of the fused compact RNN-T loss (gather+loss+grad)",
+        "value": round(bytes_step / (ms_step * 1e-3) / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16" if cfg["dtype"] == "f16" else "f32",
+        "data": "synthetic",
+        "config": {"workload": WORKLOADS[args.config], "N": N, "R": R, "V": V,
+                   "algorithmic_bytes_per_step": bytes_step, "entry": "cwarp_rnnt.transducer_loss"},
+        "pct_of_hbm_peak": round(100.0 * bytes_step / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "breakdown_ms": {"forward_call": round(fwd_ms, 4), "backward_call": round(bwd_ms, 4),
+                         "forward_nograd_call": round(nograd_ms, 4)},
+        "roofline": {"bound": "hbm", "kernel": "k_grad (cwr_backward)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic("k_grad", args.config)},
+    }
+
+    if not args.no_cpu:
+        g_all = pkg.rnnt_backward(xd, lx, y, ly, 0, st, go, out=out)
+        torch.cuda.synchronize()
+        dev_out = {"costs": costs.double().cpu().numpy(),
+                   "grad": lambda a, b: g_all[a:b].double().cpu().numpy()}
+        base, parity = cpu_baseline(cfg, x_cpu, args.cpu_budget, dev_out)
+        base["value"] = round(base["value"], 4)
+        result["cpu_baseline"] = base
+        result["parity"] = parity
+        try:
+            import torchaudio  # noqa: F401
+            result["cpu_baseline"]["torchaudio"] = "installed but not used by this leg"
+        except Exception:
+            result["cpu_baseline"]["torchaudio"] = "n/a (not installed)"
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
