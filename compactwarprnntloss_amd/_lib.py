@@ -28,9 +28,9 @@ _p, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int32, C.c_size_t
 SIGNATURES = {
     "cwr_version": (C.c_int, []),
     "cwr_strerror": (C.c_char_p, [C.c_int]),
-    "cwr_workspace_bytes": (_sz, [_i64, _i64]),
-    "cwr_workspace_section": (C.c_int, [_i64, _i64, C.c_int, C.POINTER(_sz), C.POINTER(_sz)]),
-    "cwr_diag_index": (_i64, [_i64, _i64, _i64, _i64]),
+    "cwr_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "cwr_workspace_section": (C.c_int, [_i64, _i64, _i64, C.c_int, C.POINTER(_sz), C.POINTER(_sz)]),
+    "cwr_lattice_slot": (_i64, [_i64, _i64, _i64, _i64]),
     "cwr_offsets": (C.c_int, [_p, _p, _i64, _i64, _p, _p, _p, _p]),
     "cwr_forward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                               _p, _sz, _p, _p, _p, _p, _p, _p, _p]),

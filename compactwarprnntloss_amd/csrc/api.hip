@@ -9,46 +9,61 @@ namespace cwr {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t lp, alpha, beta, bnd_a, bnd_b, total;
+    size_t pad_off, bnd_off, lp, alpha, beta, bnd_a, bnd_b, total;
+    i64 slot_cap, bnd_cap;
 };
 
-static Layout layout_for(i64 N, i64 R) {
-    (void)N;
+// Upper bounds, from what the host knows (N, R, max_u), of the lattice slots and boundary-stream
+// entries a batch can need: every strip adds at most (63 + 2*kRowShift) * 64 padding slots to the
+// R real cells, and a sequence has at most ceil((max_u+1)/64) strips.
+static Layout layout_for(i64 N, i64 R, i64 max_u) {
     Layout l;
-    size_t cells = (size_t)(R > 0 ? R : 0);
-    size_t bnd = (cells >> 6) + 1;
+    const i64 n = N > 0 ? N : 0, r = R > 0 ? R : 0, mu = max_u > 0 ? max_u : 0;
+    const i64 strips = (mu + 64) / 64;
+    i64 by_strips = r + n * strips * (63 + 2 * kRowShift) * 64;
+    i64 by_rows = r * (64 + 2 * kRowShift);  // each cell is also at most one full row of padding away
+    l.slot_cap = by_strips < by_rows ? by_strips : by_rows;
+    if (l.slot_cap < 0) l.slot_cap = 0;
+    l.bnd_cap = r / 64 + n * (strips - 1) * kBndPad + 1;
     size_t at = 0;
-    l.lp = at; at = align_up(at + cells * sizeof(float2));
-    l.alpha = at; at = align_up(at + cells * sizeof(double));
-    l.beta = at; at = align_up(at + cells * sizeof(double));
-    l.bnd_a = at; at = align_up(at + bnd * sizeof(double));
-    l.bnd_b = at; at = align_up(at + bnd * sizeof(double));
+    l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
+    l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
+    l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double2));
+    l.alpha = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
+    l.beta = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
+    l.bnd_a = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
+    l.bnd_b = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
     l.total = at;
     return l;
 }
 
-size_t workspace_bytes(i64 N, i64 R) { return layout_for(N, R).total; }
+size_t workspace_bytes(i64 N, i64 R, i64 max_u) { return layout_for(N, R, max_u).total; }
 
-bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, Workspace* ws) {
-    Layout l = layout_for(N, R);
+bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspace* ws) {
+    Layout l = layout_for(N, R, max_u);
     if (bytes < l.total) return false;
     char* p = static_cast<char*>(base);
-    ws->lp = reinterpret_cast<float2*>(p + l.lp);
+    ws->pad_off = reinterpret_cast<i64*>(p + l.pad_off);
+    ws->bnd_off = reinterpret_cast<i64*>(p + l.bnd_off);
+    ws->lp = reinterpret_cast<double2*>(p + l.lp);
     ws->alpha = reinterpret_cast<double*>(p + l.alpha);
     ws->beta = reinterpret_cast<double*>(p + l.beta);
     ws->bnd_a = reinterpret_cast<double*>(p + l.bnd_a);
     ws->bnd_b = reinterpret_cast<double*>(p + l.bnd_b);
+    ws->slot_cap = l.slot_cap;
+    ws->bnd_cap = l.bnd_cap;
     return true;
 }
 
-int workspace_section(i64 N, i64 R, int which, size_t* offset, size_t* bytes) {
+int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t* bytes) {
     if (!offset || !bytes) return CWR_ERR_NULL;
-    if (N < 0 || R < 0) return CWR_ERR_SHAPE;
-    Layout l = layout_for(N, R);
+    if (N < 0 || R < 0 || max_u < 0) return CWR_ERR_SHAPE;
+    Layout l = layout_for(N, R, max_u);
     switch (which) {
-        case 0: *offset = l.lp; *bytes = (size_t)R * sizeof(float2); return CWR_OK;
-        case 1: *offset = l.alpha; *bytes = (size_t)R * sizeof(double); return CWR_OK;
-        case 2: *offset = l.beta; *bytes = (size_t)R * sizeof(double); return CWR_OK;
+        case 0: *offset = l.lp; *bytes = (size_t)l.slot_cap * sizeof(double2); return CWR_OK;
+        case 1: *offset = l.alpha; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
+        case 2: *offset = l.beta; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
+        case 3: *offset = l.pad_off; *bytes = (size_t)(N + 1) * sizeof(i64); return CWR_OK;
     }
     return CWR_ERR_SHAPE;
 }
@@ -120,18 +135,18 @@ const char* cwr_strerror(int status) {
     return "unknown status";
 }
 
-size_t cwr_workspace_bytes(int64_t N, int64_t R) {
-    if (N < 0 || R < 0) return 0;
-    return workspace_bytes(N, R);
+size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u) {
+    if (N < 0 || R < 0 || max_u < 0) return 0;
+    return workspace_bytes(N, R, max_u);
 }
 
-int cwr_workspace_section(int64_t N, int64_t R, int which, size_t* offset, size_t* bytes) {
-    return workspace_section(N, R, which, offset, bytes);
+int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes) {
+    return workspace_section(N, R, max_u, which, offset, bytes);
 }
 
-int64_t cwr_diag_index(int64_t t, int64_t u, int64_t T, int64_t U) {
+int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U) {
     if (t < 0 || u < 0 || t >= T || u > U) return -1;
-    return diag_index(t, u, T, U + 1);
+    return lattice_slot(t, u, T, U + 1);
 }
 
 int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int64_t* row_off,
@@ -142,8 +157,9 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
     if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(row_off, 8) || misaligned(lab_off, 8) ||
         misaligned(status, 4))
         return CWR_ERR_ALIGN;
-    return launch_offsets(lx, ly, N, R, reinterpret_cast<i64*>(row_off), reinterpret_cast<i64*>(lab_off),
-                          status, nullptr, static_cast<hipStream_t>(stream));
+    return launch_offsets(lx, ly, N, R, 0, 0, 0, reinterpret_cast<i64*>(row_off),
+                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, status, nullptr,
+                          static_cast<hipStream_t>(stream));
 }
 
 static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
@@ -156,18 +172,18 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (max_u < 0) return CWR_ERR_SHAPE;
     if (!row_off || !lab_off || !status) return CWR_ERR_NULL;
     if (N > 0 && !costs) return CWR_ERR_NULL;
-    if (R > 0 && !workspace) return CWR_ERR_NULL;
+    if (!workspace) return CWR_ERR_NULL;
     if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
     if (R > 0 && with_grad && !grads) return CWR_ERR_NULL;
     if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
         misaligned(grads, 8) || misaligned(costs, 4) || misaligned(workspace, 256))
         return CWR_ERR_ALIGN;
     Workspace ws;
-    if (!carve_workspace(workspace, workspace_bytes_, N, R, &ws)) return CWR_ERR_SHAPE;
+    if (!carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws)) return CWR_ERR_SHAPE;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    rc = launch_offsets(lx, ly, N, R, reinterpret_cast<i64*>(row_off), reinterpret_cast<i64*>(lab_off),
-                        status, costs, s);
+    rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
+                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.bnd_off, status, costs, s);
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
@@ -194,7 +210,8 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, 
     // the fused gather still needs somewhere to put lse; it lives in the alpha slot, unused here
     Workspace ws;
     float* lse = nullptr;
-    if (workspace && carve_workspace(workspace, workspace_bytes_, N, R, &ws))
+    if (workspace && N >= 0 && R >= 0 && max_u >= 0 &&
+        carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws))
         lse = reinterpret_cast<float*>(ws.alpha);
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
                         workspace_bytes_, row_off, lab_off, status, lse, nullptr, costs, stream, false);

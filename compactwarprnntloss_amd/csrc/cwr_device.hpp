@@ -16,6 +16,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 // "no path" marker of the lattice recursions.  Finite, so that marker - marker = 0 instead of NaN.
 constexpr double kNeg = -1.0e30;
+constexpr float kLpFloor = -1.0e30f;  // gathered log-probs are clamped to this (keeps -inf logits finite)
 
 // ---------------------------------------------------------------------------------------------
 // wave64 cross-lane moves.  gfx9-family DPP controls.
@@ -105,15 +106,16 @@ __device__ __forceinline__ i64 wave_inclusive_scan(i64 v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// log(exp(a)+exp(b)) = max + log1p(exp(-|a-b|)), the form of cwarp_cuda_rnnt_kernel.cu:22-29.
+// log2(2^a + 2^b) = max + log2(1 + 2^-|a-b|): the form of cwarp_cuda_rnnt_kernel.cu:22-29 in
+// base 2, so that it maps onto the hardware exp2/log2 units without scaling multiplies.
 // The running values are kept in fp64 (a lattice of ~2000 steps reaches magnitudes of several
-// thousand, where an fp32 ulp is already 2e-4); the correction term, at most ln 2, is evaluated
-// on the fp32 exp2/log2 units from the fp32-rounded difference.
-__device__ __forceinline__ double log_sum_exp(double a, double b) {
+// thousand, where an fp32 ulp is already 2e-4); the correction term, at most 1, is evaluated in
+// fp32 from the fp32-rounded difference.
+__device__ __forceinline__ double log2_sum_exp2(double a, double b) {
     double mx = fmax(a, b);
-    float d = -fabsf((float)(a - b));
-    float e = fast_exp2(d * kLog2e);
-    return mx + (double)(fast_log2(1.0f + e) * kLn2);
+    float d = (float)(a - b);
+    float e = fast_exp2(-fabsf(d));
+    return mx + (double)fast_log2(1.0f + e);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -169,25 +171,29 @@ __device__ __forceinline__ void store_pack(T* __restrict__ p, const float (&in)[
 // ---------------------------------------------------------------------------------------------
 // layouts
 // ---------------------------------------------------------------------------------------------
-// Anti-diagonal order of a T x Up lattice: diagonals k = t+u ascending, inside a diagonal u
-// ascending.  diag_start(k) = number of cells on diagonals < k.
-__host__ __device__ __forceinline__ i64 diag_start(i64 k, i64 T, i64 Up) {
-    i64 m = T < Up ? T : Up;
-    i64 M = T < Up ? Up : T;
-    if (k <= m) return k * (k + 1) / 2;
-    if (k <= M) return m * (m + 1) / 2 + (k - m) * m;
-    i64 j = k - M;
-    return m * (m + 1) / 2 + (M - m) * m + j * (m - 1) - j * (j - 1) / 2;
+// Lattice storage (log-probs, alpha, beta).  A sequence's T x (U+1) lattice is cut into strips
+// of 64 label positions; strip s holds nl = min(64, U+1-64s) columns.  Inside a strip, cell
+// (t, u = 64s+l) is stored at row t+l+kRowShift, column l, of a dense (T+nl-1+2*kRowShift) x nl
+// array: a wave that walks the strip along its anti-diagonals touches one contiguous row per
+// step, at a constant pitch.  The rows above and below, and the two triangles of slots that hold
+// no cell, are padding.
+constexpr int kPF = 16;               // prefetch depth of the lattice walk, in rows
+constexpr int kRowShift = 2 * kPF;    // padding rows in front of (and behind) a strip
+constexpr int kBndPad = 192;          // entries a boundary stream holds beyond T
+
+__host__ __device__ __forceinline__ i64 strip_rows(i64 T, i64 nl) { return T + nl - 1 + 2 * kRowShift; }
+__host__ __device__ __forceinline__ i64 lattice_slots(i64 T, i64 Up) {
+    i64 full = (Up - 1) >> 6;  // strips before the last one are 64 wide
+    i64 nl = Up - (full << 6);
+    return full * strip_rows(T, 64) * 64 + strip_rows(T, nl) * nl;
 }
-__host__ __device__ __forceinline__ i64 diag_count(i64 k, i64 T, i64 Up) {
-    i64 hi = k < Up - 1 ? k : Up - 1;
-    i64 lo = k - (T - 1) > 0 ? k - (T - 1) : 0;
-    return hi - lo + 1;
+__host__ __device__ __forceinline__ i64 lattice_slot(i64 t, i64 u, i64 T, i64 Up) {
+    i64 s = u >> 6, l = u & 63;
+    i64 nl = Up - (s << 6) < 64 ? Up - (s << 6) : 64;
+    return s * strip_rows(T, 64) * 64 + (t + l + kRowShift) * nl + l;
 }
-__host__ __device__ __forceinline__ i64 diag_index(i64 t, i64 u, i64 T, i64 Up) {
-    i64 k = t + u;
-    i64 lo = k - (T - 1) > 0 ? k - (T - 1) : 0;
-    return diag_start(k, T, Up) + (u - lo);
+__host__ __device__ __forceinline__ i64 boundary_entries(i64 T, i64 Up) {
+    return ((Up - 1) >> 6) * (T + kBndPad);
 }
 
 // Which sequence owns compact row r, and where in its lattice the row sits.

@@ -32,22 +32,27 @@ struct Batch {
     hipStream_t stream;
 };
 
-// Scratch carved out of the caller's workspace.  Cells of a sequence are stored in anti-diagonal
-// order (see diag_index).
+// Scratch carved out of the caller's workspace.  lp / alpha / beta use the strip layout of
+// lattice_slot(); all values are base-2 logarithms.
 struct Workspace {
-    float2* lp;     // R    gathered (blank, label) log-probabilities
-    double* alpha;  // R
-    double* beta;   // R
-    double* bnd_a;  // R/64+1  alpha values handed from one 64-label strip to the next
-    double* bnd_b;  // R/64+1  same for beta
+    i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
+    i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
+    double2* lp;    // slot_cap  gathered (blank, label) log-probabilities
+    double* alpha;  // slot_cap
+    double* beta;   // slot_cap
+    double* bnd_a;  // bnd_cap   alpha values handed from one 64-label strip to the next
+    double* bnd_b;  // bnd_cap   same for beta
+    i64 slot_cap;
+    i64 bnd_cap;
 };
 
-size_t workspace_bytes(i64 N, i64 R);
-bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, Workspace* ws);
-int workspace_section(i64 N, i64 R, int which, size_t* offset, size_t* bytes);
+size_t workspace_bytes(i64 N, i64 R, i64 max_u);
+bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspace* ws);
+int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t* bytes);
 
-int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64* row_off, i64* lab_off,
-                   int* status, float* costs_or_null, hipStream_t stream);
+int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* status,
+                   float* costs_or_null, hipStream_t stream);
 int launch_gather(const Batch& b, const Workspace& ws, float* lse);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
 int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs);

@@ -18,6 +18,14 @@ namespace cwr {
 constexpr int kWavesPerBlock = 4;
 constexpr int kRowsPerWave = 64;
 
+// What the lattice walk consumes: (blank, label) log-probabilities as base-2 logarithms in fp64,
+// floored so that -inf logits stay finite.
+__device__ __forceinline__ double2 make_lp(float xb, float xl, float lse) {
+    const double b = ((double)fmaxf(xb, kLpFloor) - (double)lse) * 1.4426950408889634;
+    const double l = ((double)fmaxf(xl, kLpFloor) - (double)lse) * 1.4426950408889634;
+    return make_double2(b, l);
+}
+
 // position of column `col` inside a row that LPR lanes hold as K packs of VEC
 template <int VEC, int LPR>
 struct ColPos {
@@ -37,7 +45,8 @@ template <typename T, int LPR, int K>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
-    const i64* __restrict__ lab_off, int N, int blank, float2* __restrict__ lp,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    double2* __restrict__ lp,
     float* __restrict__ lse_out, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;  // rows per pass
@@ -52,9 +61,10 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
         const i64 r = r0 + lane;
         if (r < R) {
             const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-            if (ri.n >= 0) {
+            const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+            if (pad >= 0) {
                 my_lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-                my_dst = ri.off + diag_index(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+                my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             }
         }
     }
@@ -113,7 +123,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
         const float xl = __shfl(cl, g * LPR + pl.lane);
         if (ok && lir == 0) {
             lse_out[r] = lse;
-            if (dst >= 0) lp[dst] = make_float2(xb - lse, lab >= 0 ? xl - lse : 0.f);
+            if (dst >= 0) lp[dst] = make_lp(xb, lab >= 0 ? xl : lse, lse);
         }
     }
 }
@@ -123,7 +133,8 @@ template <typename T>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
-    const i64* __restrict__ lab_off, int N, int blank, float2* __restrict__ lp,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    double2* __restrict__ lp,
     float* __restrict__ lse_out, int* __restrict__ status) {
     const int lane = threadIdx.x & 63;
     const i64 r = (i64)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
@@ -140,12 +151,13 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     if (lane == 0) {
         lse_out[r] = lse;
         const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-        if (ri.n >= 0) {
+        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+        if (pad >= 0) {
             const int lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-            const i64 dst = ri.off + diag_index(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+            const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
-            lp[dst] = make_float2(xb - lse, xl - lse);
+            lp[dst] = make_lp(xb, xl, lse);
         }
     }
 }
@@ -155,18 +167,20 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_gather_logprob(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
-    const i64* __restrict__ lab_off, int N, int blank, float2* __restrict__ lp,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    double2* __restrict__ lp,
     int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
     const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-    if (ri.n < 0) return;
+    const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+    if (pad < 0) return;
     const int lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-    const i64 dst = ri.off + diag_index(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+    const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
     const T* row = x + r * (i64)V;
     const float xb = Elem<T>::to_f32(row[blank]);
     const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-    lp[dst] = make_float2(xb, xl);
+    lp[dst] = make_lp(xb, xl, 0.f);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -331,7 +345,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse) {
     if (b.mode == CWR_MODE_LOGPROB) {
         unsigned blocks = (unsigned)((b.R + 255) / 256);
         hipLaunchKernelGGL((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
-                           b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, b.N, b.blank, ws.lp,
+                           b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp,
                            b.status);
         return check_launch();
     }
@@ -343,7 +357,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse) {
     if (lpr == L && k == KK) {                                                                       \
         hipLaunchKernelGGL((k_gather_fused<T, L, KK>), dim3(blocks), dim3(kWavesPerBlock * 64), 0,   \
                            b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off,   \
-                           b.lab_off, b.N, b.blank, ws.lp, lse, b.status);                           \
+                           b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, b.status);                           \
         return check_launch();                                                                       \
     }
         CWR_SHAPES(CWR_CASE)
@@ -351,8 +365,8 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse) {
     }
     unsigned blocks = (unsigned)((b.R + kWavesPerBlock - 1) / kWavesPerBlock);
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks), dim3(kWavesPerBlock * 64), 0, b.stream,
-                       x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, b.N,
-                       b.blank, ws.lp, lse, b.status);
+                       x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,
+                       b.N, b.blank, ws.lp, lse, b.status);
     return check_launch();
 }
 

@@ -78,7 +78,7 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     st.row_off = meta[: N + 1]
     st.lab_off = meta[N + 1: 2 * (N + 1)]
     st.status = meta[2 * (N + 1):].view(torch.int32)
-    ws_bytes = lib.cwr_workspace_bytes(N, R)
+    ws_bytes = lib.cwr_workspace_bytes(N, R, int(max_u))
     st.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     costs = torch.empty(N, dtype=torch.float32, device=dev)
     st.lse = torch.empty(R, dtype=torch.float32, device=dev) if (fused and with_grad) else None

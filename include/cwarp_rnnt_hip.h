@@ -74,17 +74,19 @@ enum cwr_flag {
 int cwr_version(void);
 const char* cwr_strerror(int status);
 
-/* Bytes of scratch cwr_forward / cwr_loss need for a batch of N sequences and R rows.  The
- * scratch holds the gathered log-probabilities, alpha and beta (all O(R)); nothing in it is
- * needed by cwr_backward. */
-size_t cwr_workspace_bytes(int64_t N, int64_t R);
+/* Bytes of scratch cwr_forward / cwr_loss need for a batch of N sequences, R rows and at most
+ * max_u labels per sequence.  The scratch holds the gathered log-probabilities, alpha and beta
+ * (O(R) plus a per-sequence padding that grows with max_u, so pass a tight max_u); nothing in it
+ * is needed by cwr_backward.  Must be 256-byte aligned. */
+size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
 
 /* Location of alpha / beta inside the workspace after cwr_forward, for analysis tools (the
  * reference returns both, cwarp_cuda_rnnt_kernel.cu:383-384).  which: 0 = gathered log-probs
- * (float2 per cell), 1 = alpha, 2 = beta (float per cell).  Cells are stored per sequence in
- * anti-diagonal order: cell (t,u) of sequence n lives at row_off[n] + cwr_diag_index(t,u,T,U). */
-int cwr_workspace_section(int64_t N, int64_t R, int which, size_t* offset, size_t* bytes);
-int64_t cwr_diag_index(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
+ * (two fp64 per cell: blank, label), 1 = alpha, 2 = beta (one fp64 per cell), 3 = pad_off (N+1
+ * int64, -1 for a skipped sequence).  All values are base-2 logarithms (multiply by ln 2).
+ * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U). */
+int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes);
+int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
 
 /* Row and label offsets by a device prefix scan.
  *   row_off[n] = sum_{j<n} lx[j]*(ly[j]+1), n = 0..N   (N+1 entries, int64)
@@ -98,7 +100,8 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R,
  * (cwarp_cuda.cpp:84-108 -> gather_cuda_forward + cwarp_cuda_costs_with_grad).
  *   x        (R,V) of `dtype`, contiguous
  *   lx, ly   (N,) int32 frame / label counts;  y, y_stride: labels (see above)
- *   max_u    an upper bound of max(ly) known to the host (e.g. the padded label width)
+ *   max_u    an upper bound of max(ly) known to the host (e.g. the padded label width); a
+ *            sequence with more labels is skipped (cost NaN, CWR_FLAG_U_TOO_LARGE)
  * outputs
  *   row_off, lab_off (N+1) int64;  status 4 x int32
  *   lse      (R,) fp32 log-sum-exp of each row            [CWR_MODE_FUSED only, else may be NULL]
