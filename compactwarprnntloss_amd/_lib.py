@@ -33,11 +33,12 @@ SIGNATURES = {
     "cwr_lattice_slot": (_i64, [_i64, _i64, _i64, _i64]),
     "cwr_offsets": (C.c_int, [_p, _p, _i64, _i64, _p, _p, _p, _p]),
     "cwr_forward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
-                              _p, _sz, _p, _p, _p, _p, _p, _p, _p]),
+                              _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
     "cwr_loss": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                            _p, _sz, _p, _p, _p, _p, _p]),
     "cwr_backward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int,
-                               _p, _p, _p, _p, _p, _p, _p]),
+                               _p, _p, _p, _p, _p, _p, _p, _p]),
+    "cwr_rowinfo": (C.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p]),
 }
 
 _lib = None

@@ -22,6 +22,11 @@ FLAGS = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-ta
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 
+# The streaming kernels take row maxima with fmaxf; without this the compiler adds one
+# canonicalising v_max per input element to quiet signalling NaNs.
+EXTRA_FLAGS = {"rows.hip": ["-fno-honor-nans"]}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -37,7 +42,7 @@ def build(verbose: bool = True) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)

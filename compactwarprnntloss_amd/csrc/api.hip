@@ -9,7 +9,7 @@ namespace cwr {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t pad_off, bnd_off, lp, alpha, beta, bnd_a, bnd_b, total;
+    size_t pad_off, bnd_off, lp, alpha, beta, bnd_a, bnd_b, aux, total;
     i64 slot_cap, bnd_cap;
 };
 
@@ -33,6 +33,7 @@ static Layout layout_for(i64 N, i64 R, i64 max_u) {
     l.beta = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
     l.bnd_a = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
     l.bnd_b = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
+    l.aux = at; at = align_up(at + (size_t)r * 12);  // cwr_loss: row records (8 B) + lse (4 B) per row
     l.total = at;
     return l;
 }
@@ -50,6 +51,7 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
     ws->beta = reinterpret_cast<double*>(p + l.beta);
     ws->bnd_a = reinterpret_cast<double*>(p + l.bnd_a);
     ws->bnd_b = reinterpret_cast<double*>(p + l.bnd_b);
+    ws->aux = p + l.aux;
     ws->slot_cap = l.slot_cap;
     ws->bnd_cap = l.bnd_cap;
     return true;
@@ -165,8 +167,8 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
 static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
-                        int64_t* lab_off, int32_t* status, float* lse, float* grads, float* costs,
-                        void* stream, bool with_grad) {
+                        int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse, float* grads,
+                        float* costs, void* stream, bool with_grad) {
     int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
     if (rc != CWR_OK) return rc;
     if (max_u < 0) return CWR_ERR_SHAPE;
@@ -174,8 +176,9 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (N > 0 && !costs) return CWR_ERR_NULL;
     if (!workspace) return CWR_ERR_NULL;
     if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
-    if (R > 0 && with_grad && !grads) return CWR_ERR_NULL;
+    if (R > 0 && (!rowinfo || (with_grad && !grads))) return CWR_ERR_NULL;
     if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
+        misaligned(rowinfo, 8) ||
         misaligned(grads, 8) || misaligned(costs, 4) || misaligned(workspace, 256))
         return CWR_ERR_ALIGN;
     Workspace ws;
@@ -187,7 +190,7 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
-    rc = launch_gather(b, ws, lse);
+    rc = launch_gather(b, ws, lse, rowinfo);
     if (rc != CWR_OK) return rc;
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;
@@ -198,41 +201,63 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
 int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                 const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                 int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
-                int32_t* status, float* lse, float* grads, float* costs, void* stream) {
+                int32_t* status, int32_t* rowinfo, float* lse, float* grads, float* costs, void* stream) {
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
-                        workspace_bytes_, row_off, lab_off, status, lse, grads, costs, stream, true);
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, stream, true);
 }
 
 int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
              const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
              int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
              int32_t* status, float* costs, void* stream) {
-    // the fused gather still needs somewhere to put lse; it lives in the alpha slot, unused here
+    // the gather still needs somewhere to put lse and the row records: the workspace's aux section
     Workspace ws;
     float* lse = nullptr;
+    int32_t* rowinfo = nullptr;
     if (workspace && N >= 0 && R >= 0 && max_u >= 0 &&
-        carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws))
-        lse = reinterpret_cast<float*>(ws.alpha);
+        carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws)) {
+        rowinfo = reinterpret_cast<int32_t*>(ws.aux);
+        lse = reinterpret_cast<float*>(ws.aux + (size_t)R * 8);
+    }
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
-                        workspace_bytes_, row_off, lab_off, status, lse, nullptr, costs, stream, false);
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, nullptr, costs, stream,
+                        false);
 }
 
 int cwr_backward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                  const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
-                 const int64_t* row_off, const int64_t* lab_off, const float* grads, const float* lse,
-                 const float* grad_costs, void* grad_x, void* stream) {
+                 const int64_t* row_off, const int64_t* lab_off, const int32_t* rowinfo,
+                 const float* grads, const float* lse, const float* grad_costs, void* grad_x,
+                 void* stream) {
     int rc = check_common(x, mode == CWR_MODE_FUSED, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
     if (rc != CWR_OK) return rc;
-    if (!row_off || !lab_off) return CWR_ERR_NULL;
-    if (R > 0 && (!grads || !grad_x || !grad_costs)) return CWR_ERR_NULL;
+    (void)row_off;
+    (void)lab_off;
+    if (R > 0 && (!rowinfo || !grads || !grad_x || !grad_costs)) return CWR_ERR_NULL;
     if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
-    if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(grads, 8) || misaligned(lse, 4) ||
-        misaligned(grad_costs, 4) || misaligned(grad_x, elem_size(dtype)))
+    if (misaligned(rowinfo, 8) || misaligned(grads, 8) || misaligned(lse, 4) || misaligned(grad_costs, 4) ||
+        misaligned(grad_x, elem_size(dtype)))
         return CWR_ERR_ALIGN;
     // no status word here: the forward pass has already flagged bad labels
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, 0, row_off, lab_off,
                          nullptr, stream);
-    return launch_grad(b, grads, lse, grad_costs, grad_x);
+    return launch_grad(b, rowinfo, grads, lse, grad_costs, grad_x);
+}
+
+int cwr_rowinfo(const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                int64_t N, int64_t R, int64_t V, const int64_t* row_off, const int64_t* lab_off,
+                int32_t* rowinfo, void* stream) {
+    if (N < 0 || R < 0 || V < 1 || y_len < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff || V > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (R > 0 && N == 0) return CWR_ERR_SHAPE;
+    if ((N > 0 && (!lx || !ly)) || (y_len > 0 && !y) || !row_off || !lab_off || (R > 0 && !rowinfo))
+        return CWR_ERR_NULL;
+    if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(y, 4) || misaligned(row_off, 8) ||
+        misaligned(lab_off, 8) || misaligned(rowinfo, 8))
+        return CWR_ERR_ALIGN;
+    Batch b = make_batch(nullptr, CWR_F32, R, V, lx, ly, y, y_stride, y_len, N, 0, CWR_MODE_LOGPROB, 0,
+                         row_off, lab_off, nullptr, stream);
+    return launch_rowinfo(b, rowinfo);
 }
 
 }  // extern "C"

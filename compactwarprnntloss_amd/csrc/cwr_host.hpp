@@ -42,6 +42,7 @@ struct Workspace {
     double* beta;   // slot_cap
     double* bnd_a;  // bnd_cap   alpha values handed from one 64-label strip to the next
     double* bnd_b;  // bnd_cap   same for beta
+    char* aux;      // 12 R bytes  per-row outputs of the gather pass when the caller keeps none
     i64 slot_cap;
     i64 bnd_cap;
 };
@@ -53,12 +54,13 @@ int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                    i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* status,
                    float* costs_or_null, hipStream_t stream);
-int launch_gather(const Batch& b, const Workspace& ws, float* lse);
+int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo);
+int launch_rowinfo(const Batch& b, int* rowinfo);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
 int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs);
 int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs);
-int launch_grad(const Batch& b, const float* grads, const float* lse, const float* grad_costs,
-                void* grad_x);
+int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
+                const float* grad_costs, void* grad_x);
 
 inline int check_launch() {
     return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;

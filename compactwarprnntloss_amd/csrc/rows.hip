@@ -7,16 +7,110 @@
 //   cwarp_cuda.cpp:134 (zeros(R,V))                                > k_grad_*
 //   cwarp_cuda_rnnt_kernel.cu:512-521   cwarp_cuda_backward_      /
 //
-// Work split: a wave owns 64 consecutive rows.  In a preamble lane i decodes row r0+i (owning
-// sequence, label, per-row scalars); the main loop then walks the rows, LPR lanes per row, each
-// lane moving K 16-byte packs, and fetches the row's scalars from lane i with a wave permute.
+// Work split: waves are short-lived.  A wave handles one pass -- 64/LPR rows, LPR lanes per row,
+// K 16-byte packs per lane -- issues all its loads first, works out the rows' scalars while they
+// are in flight, and retires.  Workgroups are dispatched in address order, so at any moment the
+// machine streams one compact window of the tensor; measured on MI355X this sustains 6.2-7.0 TB/s
+// where waves that loop over many rows stay near 5.1 TB/s.
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
 namespace cwr {
 
 constexpr int kWavesPerBlock = 4;
-constexpr int kRowsPerWave = 64;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+template <bool NT>
+__device__ __forceinline__ v4i load_raw(const void* p) {
+    const v4i* q = static_cast<const v4i*>(p);
+    return NT ? __builtin_nontemporal_load(q) : *q;
+}
+template <bool NT>
+__device__ __forceinline__ void store_raw(void* p, v4i v) {
+    v4i* q = static_cast<v4i*>(p);
+    if (NT) __builtin_nontemporal_store(v, q); else *q = v;
+}
+
+// 16-byte pack <-> VEC fp32 values
+template <typename T> struct Pack;
+template <> struct Pack<float> {
+    static __device__ __forceinline__ void unpack(v4i r, float (&o)[4]) {
+        o[0] = __int_as_float(r.x); o[1] = __int_as_float(r.y); o[2] = __int_as_float(r.z); o[3] = __int_as_float(r.w);
+    }
+    static __device__ __forceinline__ v4i pack(const float (&i)[4]) {
+        v4i r = {__float_as_int(i[0]), __float_as_int(i[1]), __float_as_int(i[2]), __float_as_int(i[3])};
+        return r;
+    }
+    static __device__ __forceinline__ v4i neg_inf() {
+        v4i r = {(int)0xff800000, (int)0xff800000, (int)0xff800000, (int)0xff800000};
+        return r;
+    }
+};
+template <> struct Pack<__half> {
+    static __device__ __forceinline__ void unpack(v4i r, float (&o)[8]) {
+        const int w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            __half2 h = *reinterpret_cast<const __half2*>(&w[j]);
+            float2 f = __half22float2(h);
+            o[2 * j] = f.x; o[2 * j + 1] = f.y;
+        }
+    }
+    static __device__ __forceinline__ v4i pack(const float (&i)[8]) {
+        int w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            __half2 h = __floats2half2_rn(i[2 * j], i[2 * j + 1]);
+            w[j] = *reinterpret_cast<const int*>(&h);
+        }
+        v4i r = {w[0], w[1], w[2], w[3]};
+        return r;
+    }
+    static __device__ __forceinline__ v4i neg_inf() {
+        v4i r = {(int)0xfc00fc00, (int)0xfc00fc00, (int)0xfc00fc00, (int)0xfc00fc00};
+        return r;
+    }
+};
+template <> struct Pack<bf16_t> {
+    static __device__ __forceinline__ void unpack(v4i r, float (&o)[8]) {
+        const int w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[2 * j] = __int_as_float(w[j] << 16);
+            o[2 * j + 1] = __int_as_float(w[j] & (int)0xffff0000);
+        }
+    }
+    static __device__ __forceinline__ v4i pack(const float (&i)[8]) {
+        int w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            unsigned lo = Elem<bf16_t>::from_f32(i[2 * j]).v, hi = Elem<bf16_t>::from_f32(i[2 * j + 1]).v;
+            w[j] = (int)(lo | (hi << 16));
+        }
+        v4i r = {w[0], w[1], w[2], w[3]};
+        return r;
+    }
+    static __device__ __forceinline__ v4i neg_inf() {
+        v4i r = {(int)0xff80ff80, (int)0xff80ff80, (int)0xff80ff80, (int)0xff80ff80};
+        return r;
+    }
+};
+template <> struct Pack<double> {
+    static __device__ __forceinline__ void unpack(v4i r, float (&o)[2]) {
+        o[0] = (float)__hiloint2double(r.y, r.x);
+        o[1] = (float)__hiloint2double(r.w, r.z);
+    }
+    static __device__ __forceinline__ v4i pack(const float (&i)[2]) {
+        double a = (double)i[0], b = (double)i[1];
+        v4i r = {__double2loint(a), __double2hiint(a), __double2loint(b), __double2hiint(b)};
+        return r;
+    }
+    static __device__ __forceinline__ v4i neg_inf() {
+        v4i r = {0, (int)0xfff00000, 0, (int)0xfff00000};
+        return r;
+    }
+};
 
 // What the lattice walk consumes: (blank, label) log-probabilities as base-2 logarithms in fp64,
 // floored so that -inf logits stay finite.
@@ -41,90 +135,120 @@ struct ColPos {
 // ---------------------------------------------------------------------------------------------
 // gather, fused log-softmax: lse[r], lp[cell] = (x[r,blank]-lse, x[r,label]-lse)
 // ---------------------------------------------------------------------------------------------
+// A row held by a lane group as K packs = K*VEC fp32 values in one register vector, so that an
+// entry at a wave-uniform position can be read or written with indexed register access
+// (s_set_gpr_idx) instead of a chain of selects.
+template <int N> struct RegVec { typedef float type __attribute__((ext_vector_type(N))); };
+
+// value of row scalar `v` held by lane `i`; i is wave-uniform when a wave works on one row at a time
+template <int LPR> __device__ __forceinline__ int lane_get(int v, int i) {
+    return LPR == 64 ? __builtin_amdgcn_readlane(v, i) : __shfl(v, i);
+}
+template <int LPR> __device__ __forceinline__ float lane_get(float v, int i) {
+    return __int_as_float(lane_get<LPR>(__float_as_int(v), i));
+}
+
+// One pass: the LPR lanes of a group hold one row as K packs; all lanes of the group return the
+// row's log-sum-exp and its blank / label entries.
 template <typename T, int LPR, int K>
+__device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, const ColPos<Elem<T>::VEC, LPR>& pb,
+                                            const int lab, float& lse, float& xb, float& xl) {
+    constexpr int VEC = Elem<T>::VEC;
+    typename RegVec<K * VEC>::type xv;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        float t[VEC];
+        Pack<T>::unpack(raw[k], t);
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) xv[k * VEC + c] = t[c];
+    }
+    float m = xv[0];
+#pragma unroll
+    for (int j = 1; j < K * VEC; ++j) m = fmaxf(m, xv[j]);
+    m = group_allreduce<LPR, OpMax>(m);
+    const float ms = m * kLog2e;
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < K * VEC; ++j) s += fast_exp2(fmaf(xv[j], kLog2e, -ms));
+    s = group_allreduce<LPR, OpSum>(s);
+    lse = fmaf(fast_log2(s), kLn2, m);
+    // pick the blank and label entries out of the registers
+    const ColPos<VEC, LPR> pl(lab < 0 ? 0 : lab);
+    float cb, cl;
+    if (LPR == 64) {
+        cb = xv[pb.k * VEC + pb.c];  // uniform positions
+        cl = xv[pl.k * VEC + pl.c];
+        xb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cb), pb.lane));
+        xl = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cl), pl.lane));
+    } else {
+        cb = xv[0];
+        cl = xv[0];
+#pragma unroll
+        for (int c = 1; c < VEC; ++c) {  // K == 1 here
+            cb = c == pb.c ? xv[c] : cb;
+            cl = c == pl.c ? xv[c] : cl;
+        }
+        xb = __shfl(cb, g * LPR + pb.lane);
+        xl = __shfl(cl, g * LPR + pl.lane);
+    }
+}
+
+// first row of this wave; wave-uniform by construction, and told so to the compiler so that the
+// row decode of a one-row wave runs on the scalar unit
+__device__ __forceinline__ i64 wave_first_row(int rows_per_wave) {
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    return ((i64)blockIdx.x * kWavesPerBlock + w) * rows_per_wave;
+}
+
+template <typename T, int LPR, int K, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp,
-    float* __restrict__ lse_out, int* __restrict__ status) {
+    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
-    constexpr int RP = 64 / LPR;  // rows per pass
+    constexpr int RP = 64 / LPR;  // rows per wave
     const int lane = threadIdx.x & 63;
-    const i64 r0 = ((i64)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * kRowsPerWave;
+    const i64 r0 = wave_first_row(RP);
     if (r0 >= R) return;
-
-    // preamble: lane i looks after row r0+i
-    int my_lab = -1;
-    i64 my_dst = -1;
-    {
-        const i64 r = r0 + lane;
-        if (r < R) {
-            const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-            const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-            if (pad >= 0) {
-                my_lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-                my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
-            }
-        }
-    }
-
     const int NV = V / VEC;
     const int g = lane / LPR, lir = lane % LPR;
+    const i64 r = r0 + g;
+    const bool ok = r < R;
+
+    // loads first (a lane without a pack reads the row's first one and discards it) ...
+    const T* row = x + (ok ? r : r0) * (i64)V;
+    v4i raw[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = lir + k * LPR;
+        raw[k] = load_raw<NT>(row + (i64)(j < NV ? j : 0) * VEC);
+    }
+    // ... then the row's place in the batch, while they are in flight
+    int lab = -1, n = -1;
+    i64 dst = -1;
+    if (ok) {
+        const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+        n = ri.n;
+        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+        if (pad >= 0) {
+            lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+            dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = lir + k * LPR;
+        if (!(ok && j < NV)) raw[k] = Pack<T>::neg_inf();
+    }
     const ColPos<VEC, LPR> pb(blank);
-#pragma unroll 1
-    for (int p = 0; p < kRowsPerWave / RP; ++p) {
-        if (r0 + (i64)p * RP >= R) break;
-        const int i = p * RP + g;
-        const i64 r = r0 + i;
-        const bool ok = r < R;
-        const int lab = __shfl(my_lab, i);
-        const i64 dst = __shfl(my_dst, i);
-        const T* row = x + r * (i64)V;
-
-        float xv[K][VEC];
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const int j = lir + k * LPR;
-            if (ok && j < NV) {
-                load_pack<T, VEC>(row + (i64)j * VEC, xv[k]);
-            } else {
-#pragma unroll
-                for (int c = 0; c < VEC; ++c) xv[k][c] = -INFINITY;
-            }
-        }
-        float m = -INFINITY;
-#pragma unroll
-        for (int k = 0; k < K; ++k)
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) m = fmaxf(m, xv[k][c]);
-        m = group_allreduce<LPR, OpMax>(m);
-        const float ms = m * kLog2e;
-        float s = 0.f;
-#pragma unroll
-        for (int k = 0; k < K; ++k)
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) s += fast_exp2(fmaf(xv[k][c], kLog2e, -ms));
-        s = group_allreduce<LPR, OpSum>(s);
-        const float lse = fmaf(fast_log2(s), kLn2, m);
-
-        // pick the blank and label entries out of the registers
-        const ColPos<VEC, LPR> pl(lab < 0 ? 0 : lab);
-        float cb = 0.f, cl = 0.f;
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) {
-                if (k == pb.k && c == pb.c) cb = xv[k][c];
-                if (k == pl.k && c == pl.c) cl = xv[k][c];
-            }
-        }
-        const float xb = __shfl(cb, g * LPR + pb.lane);
-        const float xl = __shfl(cl, g * LPR + pl.lane);
-        if (ok && lir == 0) {
-            lse_out[r] = lse;
-            if (dst >= 0) lp[dst] = make_lp(xb, lab >= 0 ? xl : lse, lse);
-        }
+    float lse, xb, xl;
+    gather_pass<T, LPR, K>(raw, g, pb, lab, lse, xb, xl);
+    if (ok && lir == 0) {
+        lse_out[r] = lse;
+        rowinfo[r] = make_int2(lab, n);
+        if (dst >= 0) lp[dst] = make_lp(xb, lab >= 0 ? xl : lse, lse);
     }
 }
 
@@ -134,10 +258,10 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp,
-    float* __restrict__ lse_out, int* __restrict__ status) {
+    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ status) {
     const int lane = threadIdx.x & 63;
-    const i64 r = (i64)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const i64 r = wave_first_row(1);
     if (r >= R) return;
     const T* row = x + r * (i64)V;
     float m = -INFINITY;
@@ -152,13 +276,15 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
         lse_out[r] = lse;
         const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
         const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+        int lab = -1;
         if (pad >= 0) {
-            const int lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+            lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
             lp[dst] = make_lp(xb, xl, lse);
         }
+        rowinfo[r] = make_int2(lab, ri.n);
     }
 }
 
@@ -168,44 +294,44 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp,
-    int* __restrict__ status) {
+    double2* __restrict__ lp, int2* __restrict__ rowinfo, int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
     const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
     const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-    if (pad < 0) return;
-    const int lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-    const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
-    const T* row = x + r * (i64)V;
-    const float xb = Elem<T>::to_f32(row[blank]);
-    const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-    lp[dst] = make_lp(xb, xl, 0.f);
+    int lab = -1;
+    if (pad >= 0) {
+        lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+        const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+        const T* row = x + r * (i64)V;
+        const float xb = Elem<T>::to_f32(row[blank]);
+        const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
+        lp[dst] = make_lp(xb, xl, 0.f);
+    }
+    rowinfo[r] = make_int2(lab, ri.n);
 }
 
 // ---------------------------------------------------------------------------------------------
 // gradient pass
 // ---------------------------------------------------------------------------------------------
+// Per-row coefficients of  grad[r,v] = softmax(x_r)[v]*cg + [v==blank]*cb + [v==label]*cl  (fused)
+// or                       grad[r,v] = 0, [blank] <- cb, [label] <- cl                       (log-prob)
 struct RowCoef {
-    float cg;   // factor of softmax(x)            (fused mode)
-    float cb;   // value added / written at blank
-    float cl;   // value added / written at label
+    float cg, cb, cl;
     float nls;  // -lse * log2(e)
     int lab;
 };
 
 template <bool FUSED>
-__device__ __forceinline__ RowCoef row_coef(i64 r, i64 R, const int* lx, const int* ly, const int* y,
-                                            i64 y_stride, i64 y_len, const i64* row_off,
-                                            const i64* lab_off, int N, int V, const float2* grads,
-                                            const float* lse, const float* grad_costs, int* status) {
+__device__ __forceinline__ RowCoef row_coef(i64 r, int N, const int2* __restrict__ rowinfo,
+                                            const float2* __restrict__ grads, const float* __restrict__ lse,
+                                            const float* __restrict__ grad_costs) {
     RowCoef rc;
     rc.cg = 0.f; rc.cb = 0.f; rc.cl = 0.f; rc.nls = 0.f; rc.lab = -1;
-    if (r >= R) return rc;
-    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-    if (ri.n < 0) return rc;
-    rc.lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-    const float go = grad_costs[ri.n];
+    const int2 info = rowinfo[r];
+    if (info.y < 0 || info.y >= N) return rc;  // the row belongs to no usable sequence
+    rc.lab = info.x;
+    const float go = grad_costs[info.y];
     const float2 g = grads[r];
     rc.cb = g.x * go;
     rc.cl = rc.lab >= 0 ? g.y * go : 0.f;
@@ -216,90 +342,91 @@ __device__ __forceinline__ RowCoef row_coef(i64 r, i64 R, const int* lx, const i
     return rc;
 }
 
-template <typename T, bool FUSED, int LPR, int K>
+// One 16-byte pack of the gradient row; `pack` is its index inside the row.
+template <typename T, bool FUSED>
+__device__ __forceinline__ v4i grad_pack(v4i in, const RowCoef& rc, int pack, int blank, int V) {
+    constexpr int VEC = Elem<T>::VEC;
+    float xv[VEC], o[VEC];
+    if (FUSED) Pack<T>::unpack(in, xv);
+    const int cb_at = blank - pack * VEC;                      // component of the blank column, if 0..VEC-1
+    const int cl_at = rc.lab >= 0 ? rc.lab - pack * VEC : -1;  // same for the label column
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+        float v = FUSED ? fast_exp2(fmaf(xv[c], kLog2e, rc.nls)) * rc.cg : 0.f;
+        if (FUSED) {
+            v += c == cb_at ? rc.cb : 0.f;
+            v += c == cl_at ? rc.cl : 0.f;
+        } else {
+            v = c == cb_at ? rc.cb : v;
+            v = c == cl_at ? rc.cl : v;  // label after blank, as the reference's scatter
+        }
+        o[c] = v;
+    }
+    return Pack<T>::pack(o);
+}
+
+// Rows of NV = 64*CH packs: a wave moves 64 consecutive packs of one row, one per lane.  The row
+// is wave-uniform, so its coefficients come through the scalar unit.
+template <typename T, bool FUSED, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_flat(
+    const T* __restrict__ x, i64 R, int V, int N, int blank, int chunks_per_row,
+    const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
+    const float* __restrict__ grad_costs, T* __restrict__ gx) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const i64 wave = wave_first_row(1);  // global wave index
+    const i64 r = wave / chunks_per_row;
+    if (r >= R) return;
+    const int pack = (int)(wave - r * chunks_per_row) * 64 + lane;
+    const i64 at = r * (i64)V + (i64)pack * VEC;
+    v4i in = {0, 0, 0, 0};
+    if (FUSED) in = load_raw<NT>(x + at);
+    const RowCoef rc = row_coef<FUSED>(r, N, rowinfo, grads, lse, grad_costs);
+    store_raw<NT>(gx + at, grad_pack<T, FUSED>(in, rc, pack, blank, V));
+}
+
+// Other packed shapes: LPR lanes per row, K packs per lane, 64/LPR rows per wave.
+template <typename T, bool FUSED, int LPR, int K, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad(
-    const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
-    const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
-    const i64* __restrict__ lab_off, int N, int blank, const float2* __restrict__ grads,
-    const float* __restrict__ lse, const float* __restrict__ grad_costs, T* __restrict__ gx,
-    int* __restrict__ status) {
+    const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
+    const float2* __restrict__ grads, const float* __restrict__ lse,
+    const float* __restrict__ grad_costs, T* __restrict__ gx) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;
     const int lane = threadIdx.x & 63;
-    const i64 r0 = ((i64)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) * kRowsPerWave;
+    const i64 r0 = wave_first_row(RP);
     if (r0 >= R) return;
-    const RowCoef mine = row_coef<FUSED>(r0 + lane, R, lx, ly, y, y_stride, y_len, row_off, lab_off, N, V,
-                                         grads, lse, grad_costs, status);
     const int NV = V / VEC;
     const int g = lane / LPR, lir = lane % LPR;
-    const ColPos<VEC, LPR> pb(blank);
-#pragma unroll 1
-    for (int p = 0; p < kRowsPerWave / RP; ++p) {
-        if (r0 + (i64)p * RP >= R) break;
-        const int i = p * RP + g;
-        const i64 r = r0 + i;
-        const bool ok = r < R;
-        const float cg = __shfl(mine.cg, i);
-        const float cb = __shfl(mine.cb, i);
-        const float cl = __shfl(mine.cl, i);
-        const float nls = __shfl(mine.nls, i);
-        const int lab = __shfl(mine.lab, i);
-        const ColPos<VEC, LPR> pl(lab < 0 ? 0 : lab);
-        const bool own_b = lir == pb.lane;
-        const bool own_l = lab >= 0 && lir == pl.lane;
-
-        float xv[K][VEC];
-        if (FUSED) {
-            const T* row = x + r * (i64)V;
-#pragma unroll
-            for (int k = 0; k < K; ++k) {
-                const int j = lir + k * LPR;
-                if (ok && j < NV) {
-                    load_pack<T, VEC>(row + (i64)j * VEC, xv[k]);
-                } else {
-#pragma unroll
-                    for (int c = 0; c < VEC; ++c) xv[k][c] = 0.f;
-                }
-            }
-        }
-        T* orow = gx + r * (i64)V;
+    const i64 r = r0 + g;
+    const bool ok = r < R;
+    const i64 rbase = (ok ? r : r0) * (i64)V;
+    v4i in[K];
+    if (FUSED) {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            float o[VEC];
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) {
-                float v = FUSED ? fast_exp2(fmaf(xv[k][c], kLog2e, nls)) * cg : 0.f;
-                if (FUSED) {
-                    if (own_b && k == pb.k && c == pb.c) v += cb;
-                    if (own_l && k == pl.k && c == pl.c) v += cl;
-                } else {
-                    if (own_b && k == pb.k && c == pb.c) v = cb;
-                    if (own_l && k == pl.k && c == pl.c) v = cl;  // label after blank
-                }
-                o[c] = v;
-            }
             const int j = lir + k * LPR;
-            if (ok && j < NV) store_pack<T, VEC>(orow + (i64)j * VEC, o);
+            in[k] = load_raw<NT>(x + rbase + (i64)(j < NV ? j : 0) * VEC);
         }
+    }
+    const RowCoef rc = row_coef<FUSED>(ok ? r : r0, N, rowinfo, grads, lse, grad_costs);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = lir + k * LPR;
+        const v4i o = grad_pack<T, FUSED>(in[k], rc, j, blank, V);
+        if (ok && j < NV) store_raw<NT>(gx + rbase + (i64)j * VEC, o);
     }
 }
 
 template <typename T, bool FUSED>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_generic(
-    const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
-    const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
-    const i64* __restrict__ lab_off, int N, int blank, const float2* __restrict__ grads,
-    const float* __restrict__ lse, const float* __restrict__ grad_costs, T* __restrict__ gx,
-    int* __restrict__ status) {
+    const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
+    const float2* __restrict__ grads, const float* __restrict__ lse,
+    const float* __restrict__ grad_costs, T* __restrict__ gx) {
     const int lane = threadIdx.x & 63;
-    const i64 r = (i64)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const i64 r = wave_first_row(1);
     if (r >= R) return;
-    RowCoef rc;
-    if (lane == 0)
-        rc = row_coef<FUSED>(r, R, lx, ly, y, y_stride, y_len, row_off, lab_off, N, V, grads, lse,
-                             grad_costs, status);
-    rc.cg = __shfl(rc.cg, 0); rc.cb = __shfl(rc.cb, 0); rc.cl = __shfl(rc.cl, 0);
-    rc.nls = __shfl(rc.nls, 0); rc.lab = __shfl(rc.lab, 0);
+    const RowCoef rc = row_coef<FUSED>(r, N, rowinfo, grads, lse, grad_costs);
     const T* row = x + r * (i64)V;
     T* orow = gx + r * (i64)V;
     for (int v = lane; v < V; v += 64) {
@@ -313,6 +440,27 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_generic(
         }
         orow[v] = Elem<T>::from_f32(o);
     }
+}
+
+// The per-row record of the backward pass, for callers that did not keep the one cwr_forward wrote.
+__global__ __launch_bounds__(256) void k_rowinfo(const int* __restrict__ lx, const int* __restrict__ ly,
+                                                 const int* __restrict__ y, i64 y_stride, i64 y_len,
+                                                 const i64* __restrict__ row_off,
+                                                 const i64* __restrict__ lab_off, int N, i64 R, int V,
+                                                 int2* __restrict__ rowinfo) {
+    const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
+    if (r >= R) return;
+    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+    const int lab = ri.n >= 0 ? fetch_label(ri, y, y_stride, y_len, lab_off, V, nullptr) : -1;
+    rowinfo[r] = make_int2(lab, ri.n);
+}
+
+int launch_rowinfo(const Batch& b, int* rowinfo) {
+    if (b.R == 0) return CWR_OK;
+    hipLaunchKernelGGL(k_rowinfo, dim3((unsigned)((b.R + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly,
+                       b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, b.N, b.R, b.V,
+                       reinterpret_cast<int2*>(rowinfo));
+    return check_launch();
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -338,93 +486,107 @@ static bool packed_ok(const void* p, int V) {
 #define CWR_SHAPES(M)                                                                     \
     M(8, 1) M(16, 1) M(32, 1) M(64, 1) M(64, 2) M(64, 4) M(64, 8) M(64, 16)
 
+// streaming (non-temporal) accesses for the (R,V) tensors
+constexpr bool kGatherNT = true;
+constexpr bool kGradNT = true;
+
+static unsigned blocks_for_waves(i64 waves) { return (unsigned)((waves + kWavesPerBlock - 1) / kWavesPerBlock); }
+
 template <typename T>
-static int gather_typed(const Batch& b, const Workspace& ws, float* lse) {
+static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* rowinfo) {
     const T* x = static_cast<const T*>(b.x);
+    int2* ri = reinterpret_cast<int2*>(rowinfo);
     if (b.R == 0) return CWR_OK;
     if (b.mode == CWR_MODE_LOGPROB) {
         unsigned blocks = (unsigned)((b.R + 255) / 256);
         hipLaunchKernelGGL((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
-                           b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp,
-                           b.status);
+                           b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,
+                           ws.lp, ri, b.status);
         return check_launch();
     }
     int lpr = 0, k = 0;
     if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
-        const i64 rows_per_block = (i64)kWavesPerBlock * kRowsPerWave;
-        unsigned blocks = (unsigned)((b.R + rows_per_block - 1) / rows_per_block);
+        const int rp = 64 / lpr;
+        unsigned blocks = blocks_for_waves((b.R + rp - 1) / rp);
 #define CWR_CASE(L, KK)                                                                              \
     if (lpr == L && k == KK) {                                                                       \
-        hipLaunchKernelGGL((k_gather_fused<T, L, KK>), dim3(blocks), dim3(kWavesPerBlock * 64), 0,   \
-                           b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off,   \
-                           b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, b.status);                           \
+        hipLaunchKernelGGL((k_gather_fused<T, L, KK, kGatherNT>), dim3(blocks),                      \
+                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y,     \
+                           b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,      \
+                           ws.lp, lse, ri, b.status);                                                \
         return check_launch();                                                                       \
     }
         CWR_SHAPES(CWR_CASE)
 #undef CWR_CASE
     }
-    unsigned blocks = (unsigned)((b.R + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks), dim3(kWavesPerBlock * 64), 0, b.stream,
-                       x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,
-                       b.N, b.blank, ws.lp, lse, b.status);
+    hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
+                       0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
+                       ws.pad_off, b.N, b.blank, ws.lp, lse, ri, b.status);
     return check_launch();
 }
 
 template <typename T, bool FUSED>
-static int grad_typed(const Batch& b, const float* grads, const float* lse, const float* grad_costs,
-                      void* grad_x) {
+static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
+                      const float* grad_costs, void* grad_x) {
     const T* x = static_cast<const T*>(b.x);
     T* gx = static_cast<T*>(grad_x);
     const float2* g2 = reinterpret_cast<const float2*>(grads);
+    const int2* ri = reinterpret_cast<const int2*>(rowinfo);
     if (b.R == 0) return CWR_OK;
     int lpr = 0, k = 0;
-    if (packed_ok<T>(grad_x, b.V) && (!FUSED || packed_ok<T>(b.x, b.V)) &&
-        pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
-        const i64 rows_per_block = (i64)kWavesPerBlock * kRowsPerWave;
-        unsigned blocks = (unsigned)((b.R + rows_per_block - 1) / rows_per_block);
+    if (packed_ok<T>(grad_x, b.V) && (!FUSED || packed_ok<T>(b.x, b.V))) {
+        const int NV = b.V / Elem<T>::VEC;
+        if (NV % 64 == 0) {
+            const int ch = NV / 64;
+            hipLaunchKernelGGL((k_grad_flat<T, FUSED, kGradNT>), dim3(blocks_for_waves(b.R * ch)),
+                               dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ch, ri, g2,
+                               lse, grad_costs, gx);
+            return check_launch();
+        }
+        if (pick_shape(NV, &lpr, &k)) {
+            const int rp = 64 / lpr;
+            unsigned blocks = blocks_for_waves((b.R + rp - 1) / rp);
 #define CWR_CASE(L, KK)                                                                              \
     if (lpr == L && k == KK) {                                                                       \
-        hipLaunchKernelGGL((k_grad<T, FUSED, L, KK>), dim3(blocks), dim3(kWavesPerBlock * 64), 0,    \
-                           b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off,   \
-                           b.lab_off, b.N, b.blank, g2, lse, grad_costs, gx, b.status);              \
+        hipLaunchKernelGGL((k_grad<T, FUSED, L, KK, kGradNT>), dim3(blocks), dim3(kWavesPerBlock * 64), \
+                           0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);     \
         return check_launch();                                                                       \
     }
-        CWR_SHAPES(CWR_CASE)
+            CWR_SHAPES(CWR_CASE)
 #undef CWR_CASE
+        }
     }
-    unsigned blocks = (unsigned)((b.R + kWavesPerBlock - 1) / kWavesPerBlock);
-    hipLaunchKernelGGL((k_grad_generic<T, FUSED>), dim3(blocks), dim3(kWavesPerBlock * 64), 0, b.stream, x,
-                       b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, b.N, b.blank,
-                       g2, lse, grad_costs, gx, b.status);
+    hipLaunchKernelGGL((k_grad_generic<T, FUSED>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64), 0,
+                       b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);
     return check_launch();
 }
 
-int launch_gather(const Batch& b, const Workspace& ws, float* lse) {
+int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo) {
     switch (b.dtype) {
-        case CWR_F32: return gather_typed<float>(b, ws, lse);
-        case CWR_F16: return gather_typed<__half>(b, ws, lse);
-        case CWR_BF16: return gather_typed<bf16_t>(b, ws, lse);
-        case CWR_F64: return gather_typed<double>(b, ws, lse);
+        case CWR_F32: return gather_typed<float>(b, ws, lse, rowinfo);
+        case CWR_F16: return gather_typed<__half>(b, ws, lse, rowinfo);
+        case CWR_BF16: return gather_typed<bf16_t>(b, ws, lse, rowinfo);
+        case CWR_F64: return gather_typed<double>(b, ws, lse, rowinfo);
     }
     return CWR_ERR_DTYPE;
 }
 
-int launch_grad(const Batch& b, const float* grads, const float* lse, const float* grad_costs,
-                void* grad_x) {
+int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
+                const float* grad_costs, void* grad_x) {
     const bool fused = b.mode == CWR_MODE_FUSED;
     switch (b.dtype) {
         case CWR_F32:
-            return fused ? grad_typed<float, true>(b, grads, lse, grad_costs, grad_x)
-                         : grad_typed<float, false>(b, grads, lse, grad_costs, grad_x);
+            return fused ? grad_typed<float, true>(b, rowinfo, grads, lse, grad_costs, grad_x)
+                         : grad_typed<float, false>(b, rowinfo, grads, lse, grad_costs, grad_x);
         case CWR_F16:
-            return fused ? grad_typed<__half, true>(b, grads, lse, grad_costs, grad_x)
-                         : grad_typed<__half, false>(b, grads, lse, grad_costs, grad_x);
+            return fused ? grad_typed<__half, true>(b, rowinfo, grads, lse, grad_costs, grad_x)
+                         : grad_typed<__half, false>(b, rowinfo, grads, lse, grad_costs, grad_x);
         case CWR_BF16:
-            return fused ? grad_typed<bf16_t, true>(b, grads, lse, grad_costs, grad_x)
-                         : grad_typed<bf16_t, false>(b, grads, lse, grad_costs, grad_x);
+            return fused ? grad_typed<bf16_t, true>(b, rowinfo, grads, lse, grad_costs, grad_x)
+                         : grad_typed<bf16_t, false>(b, rowinfo, grads, lse, grad_costs, grad_x);
         case CWR_F64:
-            return fused ? grad_typed<double, true>(b, grads, lse, grad_costs, grad_x)
-                         : grad_typed<double, false>(b, grads, lse, grad_costs, grad_x);
+            return fused ? grad_typed<double, true>(b, rowinfo, grads, lse, grad_costs, grad_x)
+                         : grad_typed<double, false>(b, rowinfo, grads, lse, grad_costs, grad_x);
     }
     return CWR_ERR_DTYPE;
 }

@@ -38,7 +38,8 @@ def _label_args(ys: torch.Tensor):
 
 class ForwardState:
     """What a forward call leaves behind for the backward pass and for inspection."""
-    __slots__ = ("row_off", "lab_off", "status", "lse", "grads", "workspace", "N", "R", "V", "mode")
+    __slots__ = ("row_off", "lab_off", "status", "rowinfo", "lse", "grads", "workspace", "N", "R", "V", "mode",
+                 "max_u")
 
 
 def _check_inputs(xs, lx, ys, ly):
@@ -73,7 +74,7 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     mode = _lib.MODE_FUSED if fused else _lib.MODE_LOGPROB
 
     st = ForwardState()
-    st.N, st.R, st.V, st.mode = N, R, V, mode
+    st.N, st.R, st.V, st.mode, st.max_u = N, R, V, mode, int(max_u)
     meta = torch.empty(2 * (N + 1) + 2, dtype=torch.int64, device=dev)
     st.row_off = meta[: N + 1]
     st.lab_off = meta[N + 1: 2 * (N + 1)]
@@ -83,6 +84,7 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     costs = torch.empty(N, dtype=torch.float32, device=dev)
     st.lse = torch.empty(R, dtype=torch.float32, device=dev) if (fused and with_grad) else None
     st.grads = torch.empty((R, 2), dtype=torch.float32, device=dev) if with_grad else None
+    st.rowinfo = torch.empty((R, 2), dtype=torch.int32, device=dev) if with_grad else None
 
     with torch.cuda.device(dev):
         common = (xs.data_ptr(), _DTYPES[xs.dtype], R, V, lx.data_ptr(), ly.data_ptr(), ys.data_ptr(),
@@ -90,7 +92,8 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
                   st.workspace.data_ptr(), ws_bytes, st.row_off.data_ptr(), st.lab_off.data_ptr(),
                   st.status.data_ptr())
         if with_grad:
-            rc = lib.cwr_forward(*common, st.lse.data_ptr() if st.lse is not None else None,
+            rc = lib.cwr_forward(*common, st.rowinfo.data_ptr(),
+                                 st.lse.data_ptr() if st.lse is not None else None,
                                  st.grads.data_ptr(), costs.data_ptr(), _stream_ptr(dev))
             _lib.check(rc, "cwr_forward")
         else:
@@ -114,7 +117,7 @@ def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torc
         rc = lib.cwr_backward(xs.data_ptr() if fused else None, _DTYPES[dtype], st.R, st.V,
                               lx.data_ptr(), ly.data_ptr(), ys.data_ptr(), y_stride, y_len, st.N,
                               int(blank), st.mode, st.row_off.data_ptr(), st.lab_off.data_ptr(),
-                              st.grads.data_ptr(), st.lse.data_ptr() if fused else None,
+                              st.rowinfo.data_ptr(), st.grads.data_ptr(), st.lse.data_ptr() if fused else None,
                               gc.data_ptr(), out.data_ptr(), _stream_ptr(dev))
         _lib.check(rc, "cwr_backward")
     return out

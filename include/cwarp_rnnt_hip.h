@@ -104,6 +104,8 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R,
  *            sequence with more labels is skipped (cost NaN, CWR_FLAG_U_TOO_LARGE)
  * outputs
  *   row_off, lab_off (N+1) int64;  status 4 x int32
+ *   rowinfo  (R,2) int32 per-row record for cwr_backward: (label of the row or -1, sequence of the
+ *            row or -1)
  *   lse      (R,) fp32 log-sum-exp of each row            [CWR_MODE_FUSED only, else may be NULL]
  *   grads    (R,2) fp32 d cost / d(blank log-prob, label log-prob) per row, as the reference's
  *            `grads` (cwarp_cuda_rnnt_kernel.cu:275-332)
@@ -112,7 +114,7 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
                 const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
                 int64_t N, int32_t blank, int mode, int64_t max_u,
                 void* workspace, size_t workspace_bytes,
-                int64_t* row_off, int64_t* lab_off, int32_t* status,
+                int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
                 float* lse, float* grads, float* costs, void* stream);
 
 /* Loss only (no gradient state).  Replaces _cwarp_rnnt_loss (cwarp_cuda.cpp:58-82 ->
@@ -132,13 +134,22 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V,
  *   CWR_MODE_FUSED:   grad_x[r,v] = g*(softmax(x_r)[v]*gamma_r + grads[r,0][v==blank]
  *                     + grads[r,1][v==label]),  gamma_r = -(grads[r,0]+grads[r,1]).
  * with g = grad_costs[n] of the row's sequence (cwarp_cuda_rnnt_kernel.cu:518-519).
+ *   rowinfo  as written by cwr_forward (or cwr_rowinfo); lx, ly, y, row_off, lab_off are accepted
+ *            for symmetry with the reference's signature and may be NULL.
  *   grad_x   (R,V) of `dtype`, fully written. */
 int cwr_backward(const void* x, int dtype, int64_t R, int64_t V,
                  const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
                  int64_t N, int32_t blank, int mode,
-                 const int64_t* row_off, const int64_t* lab_off,
+                 const int64_t* row_off, const int64_t* lab_off, const int32_t* rowinfo,
                  const float* grads, const float* lse, const float* grad_costs,
                  void* grad_x, void* stream);
+
+/* The per-row record cwr_backward reads, rebuilt from the lengths and labels, for a caller that
+ * kept `grads` but not the `rowinfo` cwr_forward wrote (the reference's backward likewise rebuilds
+ * its offsets from lx and ly, cwarp_cuda.cpp:124-129).  row_off / lab_off as from cwr_offsets. */
+int cwr_rowinfo(const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                int64_t N, int64_t R, int64_t V, const int64_t* row_off, const int64_t* lab_off,
+                int32_t* rowinfo, void* stream);
 
 #ifdef __cplusplus
 }
