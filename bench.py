@@ -86,6 +86,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU work for the baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) so that a counter run can scale "
+                         "FETCH_SIZE / WRITE_SIZE against it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path is measured on ONE GPU (every sequence is independent, so a "
@@ -111,6 +114,14 @@ def main():
     R, V, N = cfg["R"], cfg["V"], cfg["N"]
     esize = x.element_size()
     bytes_step = R * V * 3 * esize
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         x.grad = None

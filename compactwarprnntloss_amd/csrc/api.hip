@@ -24,7 +24,9 @@ static Layout layout_for(i64 N, i64 R, i64 max_u) {
     i64 by_rows = r * (64 + 2 * kRowShift);  // each cell is also at most one full row of padding away
     l.slot_cap = by_strips < by_rows ? by_strips : by_rows;
     if (l.slot_cap < 0) l.slot_cap = 0;
-    l.bnd_cap = r / 64 + n * (strips - 1) * kBndPad + 1;
+    // boundary streams: (S-1)*(T+kBndPad) per sequence, with (S-1)*64 <= U < rows of the sequence
+    const i64 bnd_by_strips = n * (strips - 1) * kBndPad, bnd_by_rows = r * (kBndPad / 64);
+    l.bnd_cap = r / 64 + (bnd_by_strips < bnd_by_rows ? bnd_by_strips : bnd_by_rows) + 1;
     size_t at = 0;
     l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));

@@ -1,0 +1,187 @@
+"""CPU-only checks of the C ABI and the host logic: the library loads, exports every symbol the
+header declares, rejects invalid calls on the host (before any HIP call, so no GPU is needed), and
+the Python entry point mirrors the reference's argument checks."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from compactwarprnntloss_amd import _lib
+from oracle import rnnt_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "cwarp_rnnt_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cwr_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_functions()
+    assert {"cwr_forward", "cwr_loss", "cwr_backward", "cwr_offsets", "cwr_rowinfo", "cwr_version",
+            "cwr_strerror", "cwr_workspace_bytes", "cwr_workspace_section", "cwr_lattice_slot"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(_lib.SIGNATURES) == set(names)
+    assert lib.cwr_version() >= 100
+
+
+def test_strerror_covers_all_codes():
+    seen = set()
+    for code in range(0, 9):
+        msg = _lib.strerror(code)
+        assert msg and msg != "unknown status"
+        seen.add(msg)
+    assert len(seen) == 9
+    assert _lib.strerror(99) == "unknown status"
+
+
+def test_workspace_size_is_monotone_and_bounded():
+    lib = _lib.load()
+    assert lib.cwr_workspace_bytes(-1, 10, 3) == 0
+    base = lib.cwr_workspace_bytes(32, 300000, 80)
+    assert base % 256 == 0
+    assert lib.cwr_workspace_bytes(32, 300000, 160) > base
+    assert lib.cwr_workspace_bytes(32, 600000, 80) > base
+    # never more than 128 slots of 32 bytes per row, whatever max_u claims
+    huge = lib.cwr_workspace_bytes(32, 1000, 10 ** 9)
+    assert huge < 1000 * 128 * 32 + 10 ** 6
+    off, nbytes = C.c_size_t(), C.c_size_t()
+    for which in range(4):
+        assert lib.cwr_workspace_section(32, 300000, 80, which, C.byref(off), C.byref(nbytes)) == 0
+        assert off.value + nbytes.value <= base and off.value % 256 == 0
+    assert lib.cwr_workspace_section(32, 300000, 80, 9, C.byref(off), C.byref(nbytes)) == 4
+
+
+def test_lattice_slot_is_a_bijection_into_the_bound():
+    """Every cell of a T x (U+1) lattice gets its own slot below lattice size, for shapes around
+    the 64-column strip width."""
+    lib = _lib.load()
+    for T, U in [(1, 0), (1, 70), (5, 3), (3, 63), (3, 64), (2, 130), (40, 65)]:
+        slots = set()
+        for t in range(T):
+            for u in range(U + 1):
+                s = lib.cwr_lattice_slot(t, u, T, U)
+                assert s >= 0
+                slots.add(s)
+        assert len(slots) == T * (U + 1)
+        strips = U // 64 + 1
+        nl = U + 1 - 64 * (strips - 1)
+        size = (strips - 1) * (T + 63 + 64) * 64 + (T + nl - 1 + 64) * nl
+        assert max(slots) < size
+        assert lib.cwr_lattice_slot(T, 0, T, U) == -1 and lib.cwr_lattice_slot(0, U + 1, T, U) == -1
+
+
+def _fake(n=1):
+    """A non-null, 256-byte aligned host address: validation never dereferences it."""
+    return 0x10000 * n
+
+
+def test_invalid_calls_are_rejected_on_the_host():
+    lib = _lib.load()
+    p = _fake
+    ok_args = dict(x=p(1), dtype=0, R=10, V=8, lx=p(2), ly=p(3), y=p(4), y_stride=3, y_len=6, N=2, blank=0,
+                   mode=1, max_u=3, ws=p(5), ws_bytes=1 << 30, row_off=p(6), lab_off=p(7), status=p(8),
+                   rowinfo=p(9), lse=p(10), grads=p(11), costs=p(12), stream=None)
+
+    def fwd(**kw):
+        a = dict(ok_args, **kw)
+        return lib.cwr_forward(a["x"], a["dtype"], a["R"], a["V"], a["lx"], a["ly"], a["y"], a["y_stride"],
+                               a["y_len"], a["N"], a["blank"], a["mode"], a["max_u"], a["ws"], a["ws_bytes"],
+                               a["row_off"], a["lab_off"], a["status"], a["rowinfo"], a["lse"], a["grads"],
+                               a["costs"], a["stream"])
+
+    assert fwd(dtype=7) == 2            # CWR_ERR_DTYPE
+    assert fwd(mode=5) == 3             # CWR_ERR_MODE
+    assert fwd(R=-1) == 4               # CWR_ERR_SHAPE
+    assert fwd(V=0) == 4
+    assert fwd(N=0) == 4                # rows without sequences
+    assert fwd(max_u=-1) == 4
+    assert fwd(blank=8) == 5            # CWR_ERR_BLANK (cwarp_rnnt/__init__.py:50)
+    assert fwd(blank=-1) == 5
+    assert fwd(x=None) == 1             # CWR_ERR_NULL
+    assert fwd(lx=None) == 1
+    assert fwd(costs=None) == 1
+    assert fwd(lse=None) == 1           # fused mode needs lse
+    assert fwd(rowinfo=None) == 1
+    assert fwd(ws=None) == 1
+    assert fwd(ws_bytes=16) == 4        # workspace too small
+    assert fwd(x=p(1) + 2) == 6         # CWR_ERR_ALIGN
+    assert fwd(ws=p(5) + 8) == 6
+    assert fwd(N=1 << 31) == 8          # CWR_ERR_TOO_LARGE
+
+    assert lib.cwr_offsets(None, None, 3, 10, p(1), p(2), p(3), None) == 1
+    assert lib.cwr_offsets(p(1), p(2), -3, 10, p(1), p(2), p(3), None) == 4
+    assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, None, p(2), p(3),
+                            p(4), p(5), None) == 1          # rowinfo missing
+    assert lib.cwr_backward(None, 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, p(1), p(2), p(3),
+                            p(4), p(5), None) == 1          # fused mode needs x
+    assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 9, 0, None, None, p(1), p(2), p(3),
+                            p(4), p(5), None) == 5
+    assert lib.cwr_rowinfo(p(1), p(2), p(3), 3, 6, 2, 10, 8, p(4), p(5), None, None) == 1
+    # R == 0 is a valid (empty) call and launches nothing that touches memory
+    assert lib.cwr_backward(None, 0, 0, 8, None, None, None, 0, 0, 0, 0, 0, None, None, None, None, None,
+                            None, None, None) == 0
+
+
+def test_entry_point_asserts_match_the_reference():
+    import cwarp_rnnt
+    x = torch.zeros((6, 4))
+    lx = torch.tensor([2], dtype=torch.int32)
+    ly = torch.tensor([2], dtype=torch.int32)
+    y = torch.tensor([[1, 2]], dtype=torch.int32)
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x, lx.long(), y, ly)          # lx must be int32
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x, lx, y.long(), ly)          # y must be int32
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x, lx, y, ly, reduction="avg")
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x, lx, y, ly, blank=4)         # blank < V
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x, lx, torch.zeros((2, 2), dtype=torch.int32), ly)  # y.size(0) == N
+    with pytest.raises(AssertionError):
+        cwarp_rnnt.transducer_loss(x.view(1, 2, 3, 4), lx, y, ly)  # compact 2-D input only
+    with pytest.raises(RuntimeError, match="CUDA"):
+        cwarp_rnnt.transducer_loss(x, lx, y, ly)                  # CPU tensors are refused, no fallback
+    assert cwarp_rnnt.__version__
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libcwarp_rnnt_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "compactwarprnntloss_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f
+    assert "oracle" not in open(os.path.join(ROOT, "cwarp_rnnt", "__init__.py")).read()
+
+
+def test_golden_fixtures_match_the_oracle():
+    """The committed fixtures (written by tests/golden/make_golden.py from the oracle) still
+    reproduce: guards the oracle against silent edits."""
+    gdir = os.path.join(ROOT, "tests", "golden")
+    files = sorted(f for f in os.listdir(gdir) if f.endswith(".npz"))
+    assert files, "no golden fixtures"
+    for f in files:
+        z = np.load(os.path.join(gdir, f))
+        mode = str(z["mode"])
+        out = orc.loss_and_grad(z["x"], z["lx"], z["y"], z["ly"], int(z["blank"]), mode, grad_out=z["grad_out"])
+        np.testing.assert_allclose(out["costs"], z["costs"], rtol=1e-12)
+        np.testing.assert_allclose(out["G"], z["G"], rtol=1e-10, atol=1e-14)
+        np.testing.assert_allclose(out["grad"], z["grad"], rtol=1e-10, atol=1e-14)
+        assert np.array_equal(orc.row_offsets(z["lx"], z["ly"]), z["row_off_i32"])

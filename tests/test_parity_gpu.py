@@ -254,3 +254,25 @@ def test_data_dependent_problems_are_flagged_not_faulted():
         cwarp_rnnt.transducer_loss(b2["x"].to(dev), torch.from_numpy(b2["lx"]).to(dev),
                                    torch.from_numpy(b2["yp"]).to(dev), torch.from_numpy(b2["ly"]).to(dev),
                                    fused_log_softmax=True, validate=True)
+
+
+# ----------------------------------------------------------------------------- golden fixtures
+def _golden_files():
+    import os
+    gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    return sorted(os.path.join(gdir, f) for f in os.listdir(gdir) if f.endswith(".npz"))
+
+
+@pytest.mark.parametrize("path", _golden_files(), ids=lambda p: p.split("/")[-1][:-4])
+def test_against_golden_fixtures(path):
+    z = np.load(path)
+    fused = str(z["mode"]) == "fused"
+    b = dict(lx=z["lx"], ly=z["ly"], yp=z["y"], yc=np.concatenate([z["y"][n, : z["ly"][n]] for n in range(len(z["lx"]))]),
+             x=torch.from_numpy(z["x"]), V=z["x"].shape[1], R=z["x"].shape[0], N=len(z["lx"]), blank=int(z["blank"]))
+    for labels in ("2d", "1d"):
+        dev = run_device(b, fused, labels, z["grad_out"])
+        assert dev["flags"] == 0
+        assert np.array_equal(dev["row_off"][:-1].astype(np.int32), z["row_off_i32"])
+        np.testing.assert_allclose(dev["costs"], z["costs"], rtol=LOSS_RTOL)
+        np.testing.assert_allclose(dev["G"], z["G"], atol=GRAD_ATOL)
+        np.testing.assert_allclose(dev["grad"], z["grad"], atol=GRAD_ATOL)
