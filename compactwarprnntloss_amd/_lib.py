@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libcwarp_rnnt_hip.so")
+# CWARP_RNNT_LIB points at a library built elsewhere (same ABI); the default is the in-tree build
+LIB_PATH = os.environ.get("CWARP_RNNT_LIB") or os.path.join(HERE, "libcwarp_rnnt_hip.so")
 
 # enum cwr_dtype / cwr_mode / cwr_flag
 F32, F16, BF16, F64 = 0, 1, 2, 3

@@ -193,11 +193,23 @@ __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, co
     }
 }
 
+// Workgroups are handed to the 8 XCDs round-robin.  With XCD_CONTIGUOUS the grid (a multiple of 8
+// workgroups) is renumbered so that each XCD walks its own contiguous eighth of the rows: the
+// small per-row outputs of neighbouring rows then meet in ONE L2 and leave it as full lines,
+// instead of as eight partial lines from eight L2s.
+template <bool XCD_CONTIGUOUS>
+__device__ __forceinline__ i64 logical_block() {
+    if (!XCD_CONTIGUOUS) return blockIdx.x;
+    const unsigned per_xcd = gridDim.x >> 3;
+    return (i64)(blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+}
+
 // first row of this wave; wave-uniform by construction, and told so to the compiler so that the
 // row decode of a one-row wave runs on the scalar unit
+template <bool XCD_CONTIGUOUS = false>
 __device__ __forceinline__ i64 wave_first_row(int rows_per_wave) {
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    return ((i64)blockIdx.x * kWavesPerBlock + w) * rows_per_wave;
+    return (logical_block<XCD_CONTIGUOUS>() * kWavesPerBlock + w) * rows_per_wave;
 }
 
 template <typename T, int LPR, int K, bool NT>
@@ -210,7 +222,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;  // rows per wave
     const int lane = threadIdx.x & 63;
-    const i64 r0 = wave_first_row(RP);
+    const i64 r0 = wave_first_row<true>(RP);
     if (r0 >= R) return;
     const int NV = V / VEC;
     const int g = lane / LPR, lir = lane % LPR;
@@ -374,7 +386,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_flat(
     const float* __restrict__ grad_costs, T* __restrict__ gx) {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & 63;
-    const i64 wave = wave_first_row(1);  // global wave index
+    const i64 wave = wave_first_row<true>(1);  // global wave index
     const i64 r = wave / chunks_per_row;
     if (r >= R) return;
     const int pack = (int)(wave - r * chunks_per_row) * 64 + lane;
@@ -507,7 +519,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     int lpr = 0, k = 0;
     if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
         const int rp = 64 / lpr;
-        unsigned blocks = blocks_for_waves((b.R + rp - 1) / rp);
+        unsigned blocks = (blocks_for_waves((b.R + rp - 1) / rp) + 7u) & ~7u;  // see logical_block
 #define CWR_CASE(L, KK)                                                                              \
     if (lpr == L && k == KK) {                                                                       \
         hipLaunchKernelGGL((k_gather_fused<T, L, KK, kGatherNT>), dim3(blocks),                      \
@@ -538,7 +550,7 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
         const int NV = b.V / Elem<T>::VEC;
         if (NV % 64 == 0) {
             const int ch = NV / 64;
-            hipLaunchKernelGGL((k_grad_flat<T, FUSED, kGradNT>), dim3(blocks_for_waves(b.R * ch)),
+            hipLaunchKernelGGL((k_grad_flat<T, FUSED, kGradNT>), dim3((blocks_for_waves(b.R * ch) + 7u) & ~7u),
                                dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ch, ri, g2,
                                lse, grad_costs, gx);
             return check_launch();
