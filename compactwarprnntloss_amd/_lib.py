@@ -15,13 +15,15 @@ LIB_PATH = os.environ.get("CWARP_RNNT_LIB") or os.path.join(HERE, "libcwarp_rnnt
 # enum cwr_dtype / cwr_mode / cwr_flag
 F32, F16, BF16, F64 = 0, 1, 2, 3
 MODE_LOGPROB, MODE_FUSED = 0, 1
-FLAG_ROWS_MISMATCH, FLAG_BAD_LENGTH, FLAG_BAD_LABEL, FLAG_FB_MISMATCH, FLAG_U_TOO_LARGE = 1, 2, 4, 8, 16
+FLAG_ROWS_MISMATCH, FLAG_BAD_LENGTH, FLAG_BAD_LABEL, FLAG_FB_MISMATCH, FLAG_U_TOO_LARGE, FLAG_INTERNAL = \
+    1, 2, 4, 8, 16, 32
 FLAG_NAMES = {
     FLAG_ROWS_MISMATCH: "sum(lx*(ly+1)) differs from the number of rows of x",
     FLAG_BAD_LENGTH: "a frame length <= 0 or a label length < 0",
     FLAG_BAD_LABEL: "a label outside [0, V)",
     FLAG_FB_MISMATCH: "forward/backward likelihood mismatch above 0.1 %",
     FLAG_U_TOO_LARGE: "a label length above the max_u given",
+    FLAG_INTERNAL: "a bounded wait inside a kernel ran out",
 }
 
 _p, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int32, C.c_size_t

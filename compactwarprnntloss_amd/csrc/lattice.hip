@@ -146,40 +146,72 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 // ---------------------------------------------------------------------------------------------
 // lattice
 // ---------------------------------------------------------------------------------------------
-// Walk one strip of nl columns and T frames: rows q = 0 .. T+nl-2 (alpha) or back (beta).
-//   alpha: r = lse(own, nbr);          own' = r + B;  nbr' = r + L     (the parents' log-probs)
-//   beta : r = lse(own + B, nbr + L);  own' = nbr' = r                 (the cell's own log-probs)
+// Walk one strip of nl columns and T frames, Q = T+nl-1 steps; step k handles row q = k (alpha)
+// or q = Q-1-k (beta) of the strip.  With a = value of the cell, B / L its blank / label log-prob:
+//   alpha: a = lse(own, nbr);  own' = a + B(t,u);    nbr' = a + L(t,u)     -> cells (t+1,u), (t,u+1)
+//   beta : a = lse(own, nbr);  own' = a + B(t-1,u);  nbr' = a + L(t,u-1)   -> cells (t-1,u), (t,u-1)
+// i.e. every cell adds the log-prob of the transition INTO its successor, so that the only
+// operations between receiving the neighbour's value and handing one's own on are those of the
+// log-sum-exp itself (beta fetches L(t,u-1) from the lane on its left one step ahead of time).
+//
 // Lanes that hold no cell at a step are not masked:
 //   - before its first cell a lane holds the "no path" marker (-1e30) in own and nbr'; it reads
 //     zeros from the padding (cleared below), so the marker survives (1e30 absorbs any sum);
-//   - the start cell is produced by seeding its lane's `own` with 0 (alpha[0][0] = lse(0, none) = 0,
-//     beta[T-1][U] = lse(0 + B, none) = B);
+//   - the start cell is produced by seeding its lane's `own` (alpha[0][0] = lse(0, none) = 0,
+//     beta[T-1][U] = lse(B, none) = B);
 //   - after its last cell a lane computes junk that no lane with a cell reads any more, and
 //     stores it into padding slots;
 //   - lanes >= nl use an offset every buffer range check rejects (loads give 0, stores vanish).
-// The value a strip hands to the next one (alpha: r + L of its last column; beta: r of its first
-// column) goes through a boundary stream indexed by row; the receiving edge lane loads it as the
-// `old` operand of the DPP shift, so it lands in the lane that has no neighbour.
-template <bool BETA, bool HAS_IN, bool HAS_OUT>
-__device__ __forceinline__ void sweep_strip(const int T, const int nl, const bool seed,
+//
+// A strip hands the values of its edge column to the next strip through a boundary stream
+// indexed by the producer's step; the receiving edge lane takes the value in as the `old` operand
+// of the DPP shift, so it lands in the lane that has no neighbour.  The stream is either a span of
+// global memory (strips walked one after the other by one wave) or a ring in LDS (strips walked
+// concurrently by one wave each, `Ring`).
+constexpr int kRing = 256;             // entries of an LDS boundary ring (a multiple of kPF)
+constexpr int kSpinLimit = 1 << 22;    // polls after which a waiting wave gives up
+
+struct Ring {
+    double* slots;   // LDS, kRing entries (+ a dummy area behind them for the lanes that hold no edge)
+    int* produced;   // LDS, steps the producer has completed (INT_MAX when it is done)
+    int* consumed;   // LDS, steps the consumer has completed
+};
+
+__device__ __forceinline__ bool wait_at_least(int* counter, int need, int* status) {
+    for (int spin = 0; spin < kSpinLimit; ++spin) {
+        if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= need) return true;
+        __builtin_amdgcn_s_sleep(2);
+    }
+    atomicOr(status, CWR_FLAG_INTERNAL);
+    return false;
+}
+
+// LDS accesses of one wave are performed in program order, so a counter written after the ring
+// slots it announces needs no hardware wait; the compiler only has to keep the order.
+__device__ __forceinline__ void keep_order() { asm volatile("" ::: "memory"); }
+
+template <bool BETA, bool HAS_IN, bool HAS_OUT, bool CONC>
+__device__ __forceinline__ void sweep_strip(const int T, const int nl, const bool seed, const int in_shift,
+                                            const int out_shift,
                                             const double2* lp_strip, double* out_strip,
-                                            const double* bnd_in, double* bnd_out) {
+                                            const double* bnd_in, double* bnd_out, const Ring rin,
+                                            const Ring rout, int* status) {
     const int lane = threadIdx.x & 63;
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
     const __amdgpu_buffer_rsrc_t r_lp = make_rsrc(lp_strip, rows * nl * 16);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * nl * 8);
-    const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, HAS_IN ? ((i64)T + kBndPad) * 8 : 0);
-    const __amdgpu_buffer_rsrc_t r_bo = make_rsrc(bnd_out, HAS_OUT ? ((i64)T + kBndPad) * 8 : 0);
+    const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, (HAS_IN && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
+    const __amdgpu_buffer_rsrc_t r_bo = make_rsrc(bnd_out, (HAS_OUT && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
     const int vo_lp = lane < nl ? lane * 16 : kOob;
     const int vo_out = lane < nl ? lane * 8 : kOob;
-    const int vo_in = lane == (BETA ? 63 : 0) ? 0 : kOob;
-    const int vo_bo = lane == (BETA ? 0 : 63) ? 0 : kOob;
+    const int in_lane = BETA ? 63 : 0, out_lane = BETA ? 0 : 63;
+    const int vo_in = lane == in_lane ? 0 : kOob;
+    const int vo_bo = lane == out_lane ? 0 : kOob;
+    // LDS: the edge lane writes the ring, every other lane a private dummy slot behind it
+    double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     const int p16 = nl * 16, p8 = nl * 8;
     constexpr int dq = BETA ? -1 : 1;
-    // index of the boundary entry relative to the row index (see kBndPad)
-    constexpr int in_shift = BETA ? 1 : 63;
-    constexpr int out_shift = BETA ? 64 : 0;
 
     // clear the triangle of padding slots this direction reads before a lane's first cell
     for (int j = 0; j < nl - 1; ++j) {
@@ -190,84 +222,166 @@ __device__ __forceinline__ void sweep_strip(const int T, const int nl, const boo
     __threadfence_block();
 
     int qi = (BETA ? Q - 1 : 0) + kRowShift;  // current row
-    double2 ring[kPF];
-    double ering[kPF];
+    double2 ring[kPF];                        // log-probs of the next kPF rows
+    double ering[kPF];                        // incoming boundary values (global stream only)
 #pragma unroll
     for (int j = 0; j < kPF; ++j) {
         ring[j] = buf_load_d2(r_lp, vo_lp, (qi + dq * j) * p16);
-        ering[j] = HAS_IN ? buf_load_d(r_in, vo_in, (qi + dq * j + in_shift) * 8) : kNeg;
+        ering[j] = (HAS_IN && !CONC) ? buf_load_d(r_in, vo_in, (j + in_shift) * 8) : kNeg;
     }
-    double own = seed ? 0.0 : kNeg;
+    // alpha: own = 0 in the seed lane; beta: own = B of the seed lane's first cell
+    double own = seed ? (BETA ? ring[0].x : 0.0) : kNeg;
     double pass = kNeg;
     double nbr = kNeg;  // without an incoming stream the edge lane keeps this marker for good
     const int nblocks = (Q + kPF - 1) / kPF;
-    for (int blk = 0; blk < nblocks; ++blk) {
+    int k0 = 0;  // first step of the block
+    for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
+        // entries [k0+in_shift, k0+kPF+in_shift) must have been produced; the ring slots of entries
+        // [k0, k0+kPF) must be free, i.e. the consumer (which reads entry i at its step
+        // i-out_shift) must be past entry k0+kPF-1-kRing
+        if (CONC && HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
+        if (CONC && HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+        if (CONC) keep_order();
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
             const double2 c = ring[j];
-            const double e = ering[j];
-            ring[j] = buf_load_d2(r_lp, vo_lp, (qi + dq * kPF) * p16);
-            if (HAS_IN) ering[j] = buf_load_d(r_in, vo_in, (qi + dq * kPF + in_shift) * 8);
+            // the log-probs of this lane's next cell (beta needs them now, alpha only to refill)
+            const double2 cn = buf_load_d2(r_lp, vo_lp, (qi + dq * kPF) * p16);
+            const double2 c1 = ring[(j + 1) % kPF];  // the step after this one
+            ring[j] = cn;
+            double e;
+            if (HAS_IN && CONC) {
+                e = rin.slots[(k0 + j + in_shift) & (kRing - 1)];
+            } else {
+                e = ering[j];
+                if (HAS_IN) ering[j] = buf_load_d(r_in, vo_in, (k0 + j + kPF + in_shift) * 8);
+            }
+            // what this cell adds for its two successors
+            double add_own, add_pass;
+            if (BETA) {
+                add_own = c1.x;                                   // B(t-1,u): this lane's next cell
+                add_pass = dpp_f64<DPP_WAVE_SHR1>(0.0, c1.y);     // L(t,u-1): the left lane's next cell
+                if (HAS_IN) e += c.y;                             // the stream carries plain beta(t,u+1)
+            } else {
+                add_own = c.x;
+                add_pass = c.y;
+            }
             const double old = HAS_IN ? e : nbr;
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(old, pass) : dpp_f64<DPP_WAVE_SHR1>(old, pass);
-            double r;
-            if (BETA) {
-                r = log2_sum_exp2(own + c.x, nbr + c.y);
-                own = r;
-                pass = r;
-            } else {
-                r = log2_sum_exp2(own, nbr);
-                own = r + c.x;
-                pass = r + c.y;
+            const double mx = fmax(own, nbr);
+            const float d = (float)(own - nbr);
+            const double l = (double)fast_log2(1.0f + fast_exp2(-fabsf(d)));
+            const double a = mx + l;
+            own = (mx + add_own) + l;
+            pass = (mx + add_pass) + l;
+            buf_store_d(r_out, vo_out, qi * p8, a);
+            if (HAS_OUT) {
+                // alpha hands on a + L(t,u) (= pass); beta hands on plain a
+                const double h = BETA ? a : pass;
+                if (CONC) ring_out[(k0 + j) & (kRing - 1)] = h;
+                else buf_store_d(r_bo, vo_bo, (k0 + j) * 8, h);
             }
-            buf_store_d(r_out, vo_out, qi * p8, r);
-            if (HAS_OUT) buf_store_d(r_bo, vo_bo, (qi + out_shift) * 8, pass);
             qi += dq;
         }
+        if (CONC) keep_order();
+        if (CONC && HAS_OUT)
+            __hip_atomic_store(rout.produced, blk + 1 == nblocks ? 0x7fffffff : k0 + kPF, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (CONC && HAS_IN)
+            __hip_atomic_store(rin.consumed, blk + 1 == nblocks ? 0x7fffffff : k0 + kPF, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
     }
 }
 
-// One wave per (sequence, direction); the strips of a sequence are walked one after the other,
-// the boundary streams between them live in global memory.
-__global__ __launch_bounds__(64) void k_lattice(const int* __restrict__ lx, const int* __restrict__ ly,
-                                                const i64* __restrict__ pad_off,
-                                                const i64* __restrict__ bnd_off, const double2* lp,
-                                                double* alpha, double* beta, double* bnd_a, double* bnd_b,
-                                                int beta_only) {
+template <bool BETA, bool CONC>
+__device__ __forceinline__ void sweep_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
+                                               int out_shift, const double2* lp, double* out, const double* bi, double* bo,
+                                               Ring rin, Ring rout, int* status) {
+    if (has_in && has_out) sweep_strip<BETA, true, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_in) sweep_strip<BETA, true, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_out) sweep_strip<BETA, false, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else sweep_strip<BETA, false, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+}
+
+// One workgroup per (sequence, direction), W waves.  A sequence of S <= W strips is walked by S
+// waves at once, each strip trailing the one that feeds it by the 64 steps the diagonal order
+// demands plus one block of kPF steps of slack; the boundary values travel through LDS rings
+// guarded by two progress counters per ring.  A wave only ever waits for the wave of the strip
+// before it (values) or after it (ring space), and strip 0 waits for nobody, so the chain always
+// drains; every wait is bounded all the same.  Longer sequences (S > W) fall back to one wave
+// walking the strips in turn with the streams in global memory.
+constexpr int kMaxWaves = 8;
+
+__global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
+    const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
+    const i64* __restrict__ bnd_off, const double2* lp, double* alpha, double* beta, double* bnd_a,
+    double* bnd_b, int beta_only, int* status) {
+    __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
+    __shared__ int s_produced[kMaxWaves];
+    __shared__ int s_consumed[kMaxWaves];
     const int n = blockIdx.x;
     const int dir = beta_only ? 1 : (int)blockIdx.y;
+    const int W = blockDim.x >> 6;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    if (threadIdx.x < kMaxWaves) {
+        s_produced[threadIdx.x] = 0;
+        s_consumed[threadIdx.x] = 0;
+    }
+    __syncthreads();
     const i64 pad = pad_off[n];
     if (pad < 0) return;
     const int T = lx[n], U = ly[n];
     const int Up = U + 1;
     const int S = (Up + 63) >> 6;
-    const int lane = threadIdx.x & 63;
     const i64 full_strip = strip_rows(T, 64) * 64;
-    double* bnd = (dir ? bnd_b : bnd_a) + bnd_off[n];
     double* out = dir ? beta : alpha;
+    const int nl_last = Up - ((S - 1) << 6);
+    Ring none;
+    none.slots = nullptr; none.produced = nullptr; none.consumed = nullptr;
+
+    if (S <= W) {
+        // position p in the order of the walk: alpha strip p, beta strip S-1-p
+        const int p = w;
+        if (p >= S) return;
+        const int s = dir ? S - 1 - p : p;
+        const int nl = s == S - 1 ? nl_last : 64;
+        const i64 base = pad + (i64)s * full_strip;
+        const bool has_in = p > 0, has_out = p < S - 1;
+        Ring rin = none, rout = none;
+        if (has_in) { rin.slots = s_ring[p - 1]; rin.produced = &s_produced[p - 1]; rin.consumed = &s_consumed[p - 1]; }
+        if (has_out) { rout.slots = s_ring[p]; rout.produced = &s_produced[p]; rout.consumed = &s_consumed[p]; }
+        if (dir == 0) {
+            sweep_dispatch<false, true>(has_in, has_out, T, nl, s == 0 && lane == 0, 63, 63, lp + base, out + base,
+                                        nullptr, nullptr, rin, rout, status);
+        } else {
+            // the strip that feeds strip s is s+1; its edge lane 0 trails its first lane by nl-1 steps
+            const int shift = (s + 1 == S - 1 ? nl_last : 64) - 1;
+            // ... and this strip's own edge lane 0 trails by nl-1, which is what its consumer sees
+            sweep_dispatch<true, true>(has_in, has_out, T, nl, s == S - 1 && lane == nl - 1, shift, nl - 1,
+                                       lp + base, out + base, nullptr, nullptr, rin, rout, status);
+        }
+        return;
+    }
+
+    if (w != 0) return;
+    double* bnd = (dir ? bnd_b : bnd_a) + bnd_off[n];
     const i64 bstride = (i64)T + kBndPad;
     for (int p = 0; p < S; ++p) {
         const int s = dir ? S - 1 - p : p;
-        const int nl = (Up - (s << 6)) < 64 ? (Up - (s << 6)) : 64;
+        const int nl = s == S - 1 ? nl_last : 64;
         const i64 base = pad + (i64)s * full_strip;
         const bool has_in = p > 0, has_out = p < S - 1;
-        // boundary j sits between strips j and j+1
+        // stream j runs between the strips at positions j and j+1 of the walk
+        const double* bi = bnd + (i64)(p > 0 ? p - 1 : 0) * bstride;
+        double* bo = bnd + (i64)p * bstride;
         if (dir == 0) {
-            const bool seed = s == 0 && lane == 0;
-            const double* bi = bnd + (i64)(s > 0 ? s - 1 : 0) * bstride;
-            double* bo = bnd + (i64)s * bstride;
-            if (has_in && has_out) sweep_strip<false, true, true>(T, nl, seed, lp + base, out + base, bi, bo);
-            else if (has_in) sweep_strip<false, true, false>(T, nl, seed, lp + base, out + base, bi, bo);
-            else if (has_out) sweep_strip<false, false, true>(T, nl, seed, lp + base, out + base, bi, bo);
-            else sweep_strip<false, false, false>(T, nl, seed, lp + base, out + base, bi, bo);
+            sweep_dispatch<false, false>(has_in, has_out, T, nl, s == 0 && lane == 0, 63, 63, lp + base, out + base,
+                                         bi, bo, none, none, status);
         } else {
-            const bool seed = s == S - 1 && lane == nl - 1;
-            const double* bi = bnd + (i64)s * bstride;
-            double* bo = bnd + (i64)(s > 0 ? s - 1 : 0) * bstride;
-            if (has_in && has_out) sweep_strip<true, true, true>(T, nl, seed, lp + base, out + base, bi, bo);
-            else if (has_in) sweep_strip<true, true, false>(T, nl, seed, lp + base, out + base, bi, bo);
-            else if (has_out) sweep_strip<true, false, true>(T, nl, seed, lp + base, out + base, bi, bo);
-            else sweep_strip<true, false, false>(T, nl, seed, lp + base, out + base, bi, bo);
+            const int shift = (s + 1 == S - 1 ? nl_last : 64) - 1;
+            sweep_dispatch<true, false>(has_in, has_out, T, nl, s == S - 1 && lane == nl - 1, shift, nl - 1,
+                                        lp + base, out + base, bi, bo, none, none, status);
         }
         __threadfence_block();
     }
@@ -275,9 +389,11 @@ __global__ __launch_bounds__(64) void k_lattice(const int* __restrict__ lx, cons
 
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
     if (b.N == 0) return CWR_OK;
+    i64 strips = (b.max_u + 64) / 64;
+    int waves = (int)(strips < 1 ? 1 : (strips > kMaxWaves ? kMaxWaves : strips));
     dim3 grid((unsigned)b.N, beta_only ? 1 : 2);
-    hipLaunchKernelGGL(k_lattice, grid, dim3(64), 0, b.stream, b.lx, b.ly, ws.pad_off, ws.bnd_off, ws.lp,
-                       ws.alpha, ws.beta, ws.bnd_a, ws.bnd_b, beta_only ? 1 : 0);
+    hipLaunchKernelGGL(k_lattice, grid, dim3(waves * 64), 0, b.stream, b.lx, b.ly, ws.pad_off, ws.bnd_off, ws.lp,
+                       ws.alpha, ws.beta, ws.bnd_a, ws.bnd_b, beta_only ? 1 : 0, b.status);
     return check_launch();
 }
 

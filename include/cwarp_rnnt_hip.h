@@ -68,7 +68,8 @@ enum cwr_flag {
     CWR_FLAG_FB_MISMATCH = 8,   /* forward and backward likelihood differ by > 0.1 % for some
                                    sequence; the cost is their mean, as in the reference
                                    (cwarp_cuda_rnnt_kernel.cu:356-364, which prints instead) */
-    CWR_FLAG_U_TOO_LARGE = 16   /* some ly exceeds the max_u given to the call */
+    CWR_FLAG_U_TOO_LARGE = 16,  /* some ly exceeds the max_u given to the call */
+    CWR_FLAG_INTERNAL = 32      /* a bounded wait inside a kernel ran out (results are invalid) */
 };
 
 int cwr_version(void);

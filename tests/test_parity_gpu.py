@@ -125,7 +125,8 @@ def test_config1_tiny(fused, labels):
 
 @pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("T,U", [(1, 0), (1, 1), (1, 7), (5, 0), (2, 1), (9, 4), (4, 9), (1, 64), (70, 62),
-                                 (70, 63), (70, 64), (33, 127), (40, 128), (20, 200), (3, 300), (300, 3)])
+                                 (70, 63), (70, 64), (33, 127), (40, 128), (20, 200), (3, 300), (300, 3),
+                                 (10, 511), (10, 512), (7, 600), (400, 130), (900, 70), (150, 200)])
 def test_edge_shapes_single_sequence(fused, T, U):
     b = make_batch([T], [U], 16, seed=T * 1000 + U, normalised=not fused)
     check_case(b, fused)
