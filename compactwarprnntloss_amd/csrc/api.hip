@@ -87,15 +87,15 @@ static bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintp
 // Checks shared by the three compute entry points.
 static int check_common(const void* x, bool need_x, int dtype, int64_t R, int64_t V, const int32_t* lx,
                         const int32_t* ly, const int32_t* y, int64_t y_len, int64_t N, int32_t blank,
-                        int mode) {
+                        int mode, bool need_lengths = true) {
     if (dtype < CWR_F32 || dtype > CWR_F64) return CWR_ERR_DTYPE;
     if (mode != CWR_MODE_LOGPROB && mode != CWR_MODE_FUSED) return CWR_ERR_MODE;
     if (N < 0 || R < 0 || V < 1 || y_len < 0) return CWR_ERR_SHAPE;
     if (N > 0x3fffffff || V > 0x3fffffff) return CWR_ERR_TOO_LARGE;
     if (R > 0 && N == 0) return CWR_ERR_SHAPE;
     if (blank < 0 || blank >= V) return CWR_ERR_BLANK;
-    if (N > 0 && (!lx || !ly)) return CWR_ERR_NULL;
-    if (y_len > 0 && !y) return CWR_ERR_NULL;
+    if (need_lengths && N > 0 && (!lx || !ly)) return CWR_ERR_NULL;
+    if (need_lengths && y_len > 0 && !y) return CWR_ERR_NULL;
     if (need_x && R > 0 && !x) return CWR_ERR_NULL;
     if (x && misaligned(x, elem_size(dtype))) return CWR_ERR_ALIGN;
     if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(y, 4)) return CWR_ERR_ALIGN;
@@ -229,13 +229,14 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, 
 int cwr_backward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                  const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                  const int64_t* row_off, const int64_t* lab_off, const int32_t* rowinfo,
-                 const float* grads, const float* lse, const float* grad_costs, void* grad_x,
-                 void* stream) {
-    int rc = check_common(x, mode == CWR_MODE_FUSED, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+                 const float* grads, const float* lse, const float* grad_costs, int64_t grad_stride,
+                 float grad_scale, void* grad_x, void* stream) {
+    int rc = check_common(x, mode == CWR_MODE_FUSED, dtype, R, V, lx, ly, y, y_len, N, blank, mode, false);
     if (rc != CWR_OK) return rc;
     (void)row_off;
     (void)lab_off;
     if (R > 0 && (!rowinfo || !grads || !grad_x || !grad_costs)) return CWR_ERR_NULL;
+    if (grad_stride != 0 && grad_stride != 1) return CWR_ERR_SHAPE;
     if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
     if (misaligned(rowinfo, 8) || misaligned(grads, 8) || misaligned(lse, 4) || misaligned(grad_costs, 4) ||
         misaligned(grad_x, elem_size(dtype)))
@@ -243,7 +244,9 @@ int cwr_backward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* 
     // no status word here: the forward pass has already flagged bad labels
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, 0, row_off, lab_off,
                          nullptr, stream);
-    return launch_grad(b, rowinfo, grads, lse, grad_costs, grad_x);
+    GradOut go;
+    go.p = grad_costs; go.stride = grad_stride; go.scale = grad_scale;
+    return launch_grad(b, rowinfo, grads, lse, go, grad_x);
 }
 
 int cwr_rowinfo(const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,

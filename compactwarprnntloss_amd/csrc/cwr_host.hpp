@@ -59,8 +59,14 @@ int launch_rowinfo(const Batch& b, int* rowinfo);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
 int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs);
 int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs);
+// d(total) / d(cost of sequence n) = p[n * stride] * scale; stride 0 broadcasts one value
+struct GradOut {
+    const float* p;
+    i64 stride;
+    float scale;
+};
 int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
-                const float* grad_costs, void* grad_x);
+                const GradOut grad_costs, void* grad_x);
 
 inline int check_launch() {
     return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;

@@ -337,13 +337,13 @@ struct RowCoef {
 template <bool FUSED>
 __device__ __forceinline__ RowCoef row_coef(i64 r, int N, const int2* __restrict__ rowinfo,
                                             const float2* __restrict__ grads, const float* __restrict__ lse,
-                                            const float* __restrict__ grad_costs) {
+                                            const GradOut grad_costs) {
     RowCoef rc;
     rc.cg = 0.f; rc.cb = 0.f; rc.cl = 0.f; rc.nls = 0.f; rc.lab = -1;
     const int2 info = rowinfo[r];
     if (info.y < 0 || info.y >= N) return rc;  // the row belongs to no usable sequence
     rc.lab = info.x;
-    const float go = grad_costs[info.y];
+    const float go = grad_costs.p[(i64)info.y * grad_costs.stride] * grad_costs.scale;
     const float2 g = grads[r];
     rc.cb = g.x * go;
     rc.cl = rc.lab >= 0 ? g.y * go : 0.f;
@@ -383,7 +383,7 @@ template <typename T, bool FUSED, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_flat(
     const T* __restrict__ x, i64 R, int V, int N, int blank, int chunks_per_row,
     const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
-    const float* __restrict__ grad_costs, T* __restrict__ gx) {
+    const GradOut grad_costs, T* __restrict__ gx) {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & 63;
     const i64 wave = wave_first_row<true>(1);  // global wave index
@@ -402,7 +402,7 @@ template <typename T, bool FUSED, int LPR, int K, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad(
     const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
     const float2* __restrict__ grads, const float* __restrict__ lse,
-    const float* __restrict__ grad_costs, T* __restrict__ gx) {
+    const GradOut grad_costs, T* __restrict__ gx) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;
     const int lane = threadIdx.x & 63;
@@ -434,7 +434,7 @@ template <typename T, bool FUSED>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_generic(
     const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
     const float2* __restrict__ grads, const float* __restrict__ lse,
-    const float* __restrict__ grad_costs, T* __restrict__ gx) {
+    const GradOut grad_costs, T* __restrict__ gx) {
     const int lane = threadIdx.x & 63;
     const i64 r = wave_first_row(1);
     if (r >= R) return;
@@ -539,7 +539,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
 
 template <typename T, bool FUSED>
 static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
-                      const float* grad_costs, void* grad_x) {
+                      const GradOut grad_costs, void* grad_x) {
     const T* x = static_cast<const T*>(b.x);
     T* gx = static_cast<T*>(grad_x);
     const float2* g2 = reinterpret_cast<const float2*>(grads);
@@ -584,7 +584,7 @@ int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo)
 }
 
 int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
-                const float* grad_costs, void* grad_x) {
+                const GradOut grad_costs, void* grad_x) {
     const bool fused = b.mode == CWR_MODE_FUSED;
     switch (b.dtype) {
         case CWR_F32:

@@ -103,13 +103,21 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
 
 
 def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torch.Tensor,
-                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Binding of cwr_backward.  Returns the (R,V) gradient in xs.dtype."""
+                  out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """Binding of cwr_backward.  Returns the (R,V) gradient in xs.dtype.
+
+    grad_costs holds d(total)/d(cost): one value per sequence, or a single value that is
+    broadcast (stride 0); `scale` multiplies it (1/N of a mean reduction)."""
     lib = _lib.load()
     dev = lx.device
     fused = st.mode == _lib.MODE_FUSED
     y_stride, y_len = _label_args(ys)
-    gc = grad_costs.to(dtype=torch.float32).contiguous()
+    gc = grad_costs
+    if gc.dtype != torch.float32 or not gc.is_contiguous():
+        gc = gc.to(dtype=torch.float32).contiguous()
+    if gc.numel() not in (1, st.N):
+        raise RuntimeError("grad_costs must hold one value or one value per sequence")
+    stride = 0 if (gc.numel() == 1 and st.N != 1) else 1
     dtype = xs.dtype
     if out is None:
         out = torch.empty((st.R, st.V), dtype=dtype, device=dev)
@@ -117,8 +125,9 @@ def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torc
         rc = lib.cwr_backward(xs.data_ptr() if fused else None, _DTYPES[dtype], st.R, st.V,
                               lx.data_ptr(), ly.data_ptr(), ys.data_ptr(), y_stride, y_len, st.N,
                               int(blank), st.mode, st.row_off.data_ptr(), st.lab_off.data_ptr(),
-                              st.rowinfo.data_ptr(), st.grads.data_ptr(), st.lse.data_ptr() if fused else None,
-                              gc.data_ptr(), out.data_ptr(), _stream_ptr(dev))
+                              st.rowinfo.data_ptr(), st.grads.data_ptr(),
+                              st.lse.data_ptr() if fused else None, gc.data_ptr(), stride, float(scale),
+                              out.data_ptr(), _stream_ptr(dev))
         _lib.check(rc, "cwr_backward")
     return out
 
@@ -131,10 +140,13 @@ def _raise_on_flags(st: ForwardState):
 
 
 class _TransLoss(torch.autograd.Function):
-    """cwarp_rnnt/__init__.py:10-29: gradient path when xs requires grad, beta-only path otherwise."""
+    """cwarp_rnnt/__init__.py:10-29: gradient path when xs requires grad, beta-only path otherwise.
+    The reduction (cwarp_rnnt/__init__.py:66-71) is part of the node, so that the backward pass
+    receives one scalar for 'mean' / 'sum' and folds it (and the 1/N) into the gradient kernel
+    instead of materialising an expanded per-sequence tensor."""
 
     @staticmethod
-    def forward(ctx: Any, xs, lx, ys, ly, blank, fused, max_u, validate):
+    def forward(ctx: Any, xs, lx, ys, ly, blank, fused, max_u, validate, reduction):
         need_grad = xs.requires_grad
         costs, st = rnnt_forward(xs, lx, ys, ly, blank, fused, max_u, with_grad=need_grad)
         if validate:
@@ -143,14 +155,22 @@ class _TransLoss(torch.autograd.Function):
             st.workspace = None  # alpha / beta are not needed again
             ctx.state = st
             ctx.blank = blank
+            ctx.reduction = reduction
             ctx.save_for_backward(xs, lx, ys, ly)
-        return costs if xs.dtype in (torch.float16, torch.bfloat16) else costs.to(xs.dtype)
+        if xs.dtype not in (torch.float16, torch.bfloat16):
+            costs = costs.to(xs.dtype)
+        if reduction == "mean":
+            return costs.mean()
+        if reduction == "sum":
+            return costs.sum()
+        return costs
 
     @staticmethod
     def backward(ctx: Any, grad_outputs):
         xs, lx, ys, ly = ctx.saved_tensors
-        grad_input = rnnt_backward(xs, lx, ys, ly, ctx.blank, ctx.state, grad_outputs)
-        return grad_input, None, None, None, None, None, None, None
+        scale = 1.0 / ctx.state.N if ctx.reduction == "mean" else 1.0
+        grad_input = rnnt_backward(xs, lx, ys, ly, ctx.blank, ctx.state, grad_outputs, scale=scale)
+        return grad_input, None, None, None, None, None, None, None, None
 
 
 def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torch.Tensor, blank: int = 0,
@@ -177,13 +197,7 @@ def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torc
     # x: (STU, V)
     assert x.dim() == 2, "input must be compact: (sum_i T_i*(U_i+1), V)"
 
-    costs = _TransLoss.apply(x, lx, y, ly, blank, bool(fused_log_softmax), max_u, bool(validate))
-
-    if reduction == "mean":
-        return costs.mean()
-    elif reduction == "sum":
-        return costs.sum()
-    elif reduction == "none" or reduction is None:
-        return costs
-    else:
+    if reduction not in ("mean", "sum", "none", None):
         raise ValueError
+    return _TransLoss.apply(x, lx, y, ly, blank, bool(fused_log_softmax), max_u, bool(validate),
+                            reduction if reduction in ("mean", "sum") else "none")

@@ -134,7 +134,10 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V,
  *                     (label written after blank, cwarp_cuda_gather_kernel.cu:70-73); x unused.
  *   CWR_MODE_FUSED:   grad_x[r,v] = g*(softmax(x_r)[v]*gamma_r + grads[r,0][v==blank]
  *                     + grads[r,1][v==label]),  gamma_r = -(grads[r,0]+grads[r,1]).
- * with g = grad_costs[n] of the row's sequence (cwarp_cuda_rnnt_kernel.cu:518-519).
+ * with g = grad_costs[n*grad_stride]*grad_scale for the row's sequence n
+ * (cwarp_cuda_rnnt_kernel.cu:518-519).  grad_stride is 1 for a per-sequence gradient or 0 to
+ * broadcast grad_costs[0] (what a mean / sum reduction hands back), grad_scale folds the 1/N of a
+ * mean reduction in, so that neither needs a kernel of its own.
  *   rowinfo  as written by cwr_forward (or cwr_rowinfo); lx, ly, y, row_off, lab_off are accepted
  *            for symmetry with the reference's signature and may be NULL.
  *   grad_x   (R,V) of `dtype`, fully written. */
@@ -143,7 +146,7 @@ int cwr_backward(const void* x, int dtype, int64_t R, int64_t V,
                  int64_t N, int32_t blank, int mode,
                  const int64_t* row_off, const int64_t* lab_off, const int32_t* rowinfo,
                  const float* grads, const float* lse, const float* grad_costs,
-                 void* grad_x, void* stream);
+                 int64_t grad_stride, float grad_scale, void* grad_x, void* stream);
 
 /* The per-row record cwr_backward reads, rebuilt from the lengths and labels, for a caller that
  * kept `grads` but not the `rowinfo` cwr_forward wrote (the reference's backward likewise rebuilds

@@ -120,15 +120,17 @@ def test_invalid_calls_are_rejected_on_the_host():
     assert lib.cwr_offsets(None, None, 3, 10, p(1), p(2), p(3), None) == 1
     assert lib.cwr_offsets(p(1), p(2), -3, 10, p(1), p(2), p(3), None) == 4
     assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, None, p(2), p(3),
-                            p(4), p(5), None) == 1          # rowinfo missing
+                            p(4), 1, 1.0, p(5), None) == 1          # rowinfo missing
     assert lib.cwr_backward(None, 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, p(1), p(2), p(3),
-                            p(4), p(5), None) == 1          # fused mode needs x
+                            p(4), 1, 1.0, p(5), None) == 1          # fused mode needs x
     assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 9, 0, None, None, p(1), p(2), p(3),
-                            p(4), p(5), None) == 5
+                            p(4), 1, 1.0, p(5), None) == 5
+    assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, p(1), p(2), p(3),
+                            p(4), 2, 1.0, p(5), None) == 4          # grad_stride is 0 or 1
     assert lib.cwr_rowinfo(p(1), p(2), p(3), 3, 6, 2, 10, 8, p(4), p(5), None, None) == 1
     # R == 0 is a valid (empty) call and launches nothing that touches memory
     assert lib.cwr_backward(None, 0, 0, 8, None, None, None, 0, 0, 0, 0, 0, None, None, None, None, None,
-                            None, None, None) == 0
+                            None, 1, 1.0, None, None) == 0
 
 
 def test_entry_point_asserts_match_the_reference():
