@@ -150,7 +150,7 @@ template <int LPR> __device__ __forceinline__ float lane_get(float v, int i) {
 
 // One pass: the LPR lanes of a group hold one row as K packs; all lanes of the group return the
 // row's log-sum-exp and its blank / label entries.
-template <typename T, int LPR, int K>
+template <typename T, int LPR, int K, bool EXTRACT = true>
 __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, const ColPos<Elem<T>::VEC, LPR>& pb,
                                             const int lab, float& lse, float& xb, float& xl) {
     constexpr int VEC = Elem<T>::VEC;
@@ -172,6 +172,7 @@ __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, co
     for (int j = 0; j < K * VEC; ++j) s += fast_exp2(fmaf(xv[j], kLog2e, -ms));
     s = group_allreduce<LPR, OpSum>(s);
     lse = fmaf(fast_log2(s), kLn2, m);
+    if (!EXTRACT) return;
     // pick the blank and label entries out of the registers
     const ColPos<VEC, LPR> pl(lab < 0 ? 0 : lab);
     float cb, cl;
@@ -212,55 +213,179 @@ __device__ __forceinline__ i64 wave_first_row(int rows_per_wave) {
     return (logical_block<XCD_CONTIGUOUS>() * kWavesPerBlock + w) * rows_per_wave;
 }
 
-template <typename T, int LPR, int K, bool NT>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused(
+// Rows of at least 4 KiB (a whole wave per row, K >= 4 packs per lane): one row per wave.  The
+// row is wave-uniform, so its decode runs on the scalar unit beside the vector work.
+template <typename T, int K, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
     double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
-    constexpr int RP = 64 / LPR;  // rows per wave
+    // beyond 32 values per lane the register vector would be indexed through scratch memory:
+    // the two entries are then read back from the row itself (it has just been fetched)
+    constexpr bool kFromRegs = K * VEC <= 32;
     const int lane = threadIdx.x & 63;
-    const i64 r0 = wave_first_row<true>(RP);
-    if (r0 >= R) return;
+    const i64 r = wave_first_row<true>(1);
+    if (r >= R) return;
     const int NV = V / VEC;
-    const int g = lane / LPR, lir = lane % LPR;
-    const i64 r = r0 + g;
-    const bool ok = r < R;
 
     // loads first (a lane without a pack reads the row's first one and discards it) ...
-    const T* row = x + (ok ? r : r0) * (i64)V;
+    const T* row = x + r * (i64)V;
     v4i raw[K];
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int j = lir + k * LPR;
+        const int j = lane + k * 64;
         raw[k] = load_raw<NT>(row + (i64)(j < NV ? j : 0) * VEC);
     }
     // ... then the row's place in the batch, while they are in flight
-    int lab = -1, n = -1;
+    int lab = -1;
     i64 dst = -1;
-    if (ok) {
-        const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-        n = ri.n;
-        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-        if (pad >= 0) {
-            lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-            dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
-        }
+    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+    const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+    if (pad >= 0) {
+        lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+        dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+    }
+    float xb = 0.f, xl = 0.f;
+    if (!kFromRegs) {
+        xb = Elem<T>::to_f32(row[blank]);
+        xl = Elem<T>::to_f32(row[lab < 0 ? 0 : lab]);
     }
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int j = lir + k * LPR;
-        if (!(ok && j < NV)) raw[k] = Pack<T>::neg_inf();
-    }
-    const ColPos<VEC, LPR> pb(blank);
-    float lse, xb, xl;
-    gather_pass<T, LPR, K>(raw, g, pb, lab, lse, xb, xl);
-    if (ok && lir == 0) {
+    for (int k = 0; k < K; ++k)
+        if (lane + k * 64 >= NV) raw[k] = Pack<T>::neg_inf();
+    const ColPos<VEC, 64> pb(blank);
+    float lse, rb, rl;
+    gather_pass<T, 64, K, kFromRegs>(raw, 0, pb, lab, lse, rb, rl);
+    if (kFromRegs) { xb = rb; xl = rl; }
+    if (lane == 0) {
         lse_out[r] = lse;
-        rowinfo[r] = make_int2(lab, n);
+        rowinfo[r] = make_int2(lab, ri.n);
         if (dst >= 0) lp[dst] = make_lp(xb, lab >= 0 ? xl : lse, lse);
+    }
+}
+
+// The per-sequence tables of a batch of at most 64 sequences, sequence l in lane l, so that a
+// lane can look its row's sequence up with cross-lane reads instead of dependent memory loads.
+struct SeqTables {
+    i64 off, pad, lab;
+    int T, U;
+};
+
+__device__ __forceinline__ i64 shfl_i64(i64 v, int src) {
+    int lo = __shfl((int)(v & 0xffffffffLL), src), hi = __shfl((int)(v >> 32), src);
+    return ((i64)hi << 32) | (i64)(unsigned)lo;
+}
+
+// Smaller rows: a wave takes NP passes of 64/LPR rows (about 4 KiB in all), issues every load up
+// front, and lane i decodes row r0+i meanwhile.
+template <typename T, int LPR, int K, int NP, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
+    const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
+    const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ status) {
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int RP = 64 / LPR;   // rows per pass
+    constexpr int ROWS = RP * NP;  // rows per wave
+    static_assert(ROWS <= 64 && K * VEC <= 32, "shape not meant for this kernel");
+    const int lane = threadIdx.x & 63;
+    const i64 r0 = wave_first_row<true>(ROWS);
+    if (r0 >= R) return;
+    const int NV = V / VEC;
+    const int g = lane / LPR, lir = lane % LPR;
+
+    v4i raw[NP][K];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const i64 r = r0 + p * RP + g;
+        const T* row = x + (r < R ? r : r0) * (i64)V;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int j = lir + k * LPR;
+            raw[p][k] = load_raw<NT>(row + (i64)(j < NV ? j : 0) * VEC);
+        }
+    }
+
+    // lane i decodes row r0+i
+    const i64 r = r0 + lane;
+    const bool mine = lane < ROWS && r < R;
+    RowInfo ri;
+    ri.n = -1; ri.t = 0; ri.u = 0; ri.T = 0; ri.U = 0; ri.off = 0;
+    i64 pad = -1, labbase = 0;
+    if (N <= 64) {
+        SeqTables tb;
+        tb.off = 0x7fffffffffffffffLL; tb.pad = -1; tb.lab = 0; tb.T = 0; tb.U = 0;
+        if (lane < N) {
+            tb.off = row_off[lane]; tb.pad = pad_off[lane]; tb.lab = lab_off[lane];
+            tb.T = lx[lane]; tb.U = ly[lane];
+        }
+        const unsigned long long m = __ballot(tb.off <= r0);
+        int n = m ? 63 - __clzll((long long)m) : 0;  // sequence of r0; later rows step over boundaries
+        const i64 r_last = r0 + ROWS - 1;
+        for (int j = n + 1; j < N; ++j) {
+            const i64 oj = shfl_i64(tb.off, j);
+            if (oj > r_last) break;
+            n += (mine && oj <= r) ? 1 : 0;
+        }
+        const i64 off = shfl_i64(tb.off, n);
+        pad = shfl_i64(tb.pad, n);
+        labbase = shfl_i64(tb.lab, n);
+        const int T_ = __shfl(tb.T, n), U_ = __shfl(tb.U, n);
+        const i64 rem = r - off;
+        if (mine && T_ > 0 && U_ >= 0 && rem >= 0 && rem < (i64)T_ * (U_ + 1)) {
+            ri.n = n; ri.T = T_; ri.U = U_; ri.off = off;
+            if ((i64)T_ * (U_ + 1) < 0x7fffffffLL) {
+                const unsigned q = (unsigned)rem / (unsigned)(U_ + 1);
+                ri.t = (int)q;
+                ri.u = (int)((unsigned)rem - q * (unsigned)(U_ + 1));
+            } else {
+                ri.t = (int)(rem / (U_ + 1));
+                ri.u = (int)(rem - (i64)ri.t * (U_ + 1));
+            }
+        }
+    } else if (mine) {
+        ri = decode_row(r, R, row_off, lx, ly, N);
+        if (ri.n >= 0) { pad = pad_off[ri.n]; labbase = lab_off[ri.n]; }
+    }
+    int my_lab = -1;
+    i64 my_dst = -1;
+    if (ri.n >= 0 && pad >= 0) {
+        if (ri.u < ri.U) {
+            const i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : labbase) + ri.u;
+            const int l = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
+            if (l < 0 || l >= V) atomicOr(status, CWR_FLAG_BAD_LABEL); else my_lab = l;
+        }
+        my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+    }
+
+    const ColPos<VEC, LPR> pb(blank);
+    float res_lse = 0.f, res_b = 0.f, res_l = 0.f;  // results of row r0+i, parked in lane i
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const bool ok = r0 + p * RP + g < R;
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+            if (!(ok && lir + k * LPR < NV)) raw[p][k] = Pack<T>::neg_inf();
+        const int lab = __shfl(my_lab, p * RP + g);
+        float lse, xb, xl;
+        gather_pass<T, LPR, K>(raw[p], g, pb, lab, lse, xb, xl);
+        const int src = (lane % RP) * LPR;  // lane i = p*RP + j wants the row of group j
+        lse = __shfl(lse, src);
+        xb = __shfl(xb, src);
+        xl = __shfl(xl, src);
+        const bool here = lane / RP == p;
+        res_lse = here ? lse : res_lse;
+        res_b = here ? xb : res_b;
+        res_l = here ? xl : res_l;
+    }
+    if (mine) {
+        lse_out[r] = res_lse;
+        rowinfo[r] = make_int2(my_lab, ri.n);
+        if (my_dst >= 0) lp[my_dst] = make_lp(res_b, my_lab >= 0 ? res_l : res_lse, res_lse);
     }
 }
 
@@ -518,18 +643,28 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     }
     int lpr = 0, k = 0;
     if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
-        const int rp = 64 / lpr;
-        unsigned blocks = (blocks_for_waves((b.R + rp - 1) / rp) + 7u) & ~7u;  // see logical_block
-#define CWR_CASE(L, KK)                                                                              \
-    if (lpr == L && k == KK) {                                                                       \
-        hipLaunchKernelGGL((k_gather_fused<T, L, KK, kGatherNT>), dim3(blocks),                      \
-                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y,     \
-                           b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,      \
-                           ws.lp, lse, ri, b.status);                                                \
+#define CWR_ARGS x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,   \
+                 b.blank, ws.lp, lse, ri, b.status
+        // grids are multiples of 8 workgroups, see logical_block
+#define CWR_ROW(KK)                                                                                  \
+    if (lpr == 64 && k == KK) {                                                                      \
+        hipLaunchKernelGGL((k_gather_row<T, KK, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u), \
+                           dim3(kWavesPerBlock * 64), 0, b.stream, CWR_ARGS);                        \
         return check_launch();                                                                       \
     }
-        CWR_SHAPES(CWR_CASE)
-#undef CWR_CASE
+#define CWR_ROWS(L, KK, NP)                                                                          \
+    if (lpr == L && k == KK) {                                                                       \
+        const int rows = (64 / L) * NP;                                                              \
+        hipLaunchKernelGGL((k_gather_rows<T, L, KK, NP, kGatherNT>),                                 \
+                           dim3((blocks_for_waves((b.R + rows - 1) / rows) + 7u) & ~7u),             \
+                           dim3(kWavesPerBlock * 64), 0, b.stream, CWR_ARGS);                        \
+        return check_launch();                                                                       \
+    }
+        CWR_ROW(4) CWR_ROW(8) CWR_ROW(16)
+        CWR_ROWS(8, 1, 4) CWR_ROWS(16, 1, 4) CWR_ROWS(32, 1, 4) CWR_ROWS(64, 1, 4) CWR_ROWS(64, 2, 2)
+#undef CWR_ROW
+#undef CWR_ROWS
+#undef CWR_ARGS
     }
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
