@@ -196,7 +196,7 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (rc != CWR_OK) return rc;
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;
-    if (with_grad) return launch_fill(b, ws, grads, costs);
+    if (with_grad) return launch_fill(b, ws, rowinfo, grads, costs);
     return launch_cost_from_beta(b, ws, costs);
 }
 

@@ -204,24 +204,18 @@ struct RowInfo {
     i64 off;  // row_off[n]
 };
 
-__device__ __forceinline__ RowInfo decode_row(i64 r, i64 R, const i64* __restrict__ row_off,
-                                              const int* __restrict__ lx, const int* __restrict__ ly,
-                                              int N) {
+// Where row r sits inside sequence n.
+__device__ __forceinline__ RowInfo place_row(i64 r, int n, i64 R, const i64* __restrict__ row_off,
+                                             const int* __restrict__ lx, const int* __restrict__ ly) {
     RowInfo ri;
     ri.n = -1; ri.t = 0; ri.u = 0; ri.T = 0; ri.U = 0; ri.off = 0;
-    if (N <= 0) return ri;
-    int lo = 0, hi = N - 1;
-    while (lo < hi) {  // last n with row_off[n] <= r (skips empty sequences)
-        int mid = (lo + hi + 1) >> 1;
-        if (row_off[mid] <= r) lo = mid; else hi = mid - 1;
-    }
-    i64 off = row_off[lo];
-    int T = lx[lo], U = ly[lo];
+    const i64 off = row_off[n];
+    const int T = lx[n], U = ly[n];
     if (T <= 0 || U < 0) return ri;
-    i64 cells = (i64)T * (i64)(U + 1);
-    i64 rem = r - off;
+    const i64 cells = (i64)T * (i64)(U + 1);
+    const i64 rem = r - off;
     if (rem < 0 || rem >= cells || off + cells > R) return ri;
-    ri.n = lo; ri.T = T; ri.U = U; ri.off = off;
+    ri.n = n; ri.T = T; ri.U = U; ri.off = off;
     if (cells < 0x7fffffffLL) {
         unsigned q = (unsigned)rem / (unsigned)(U + 1);
         ri.t = (int)q;
@@ -231,6 +225,22 @@ __device__ __forceinline__ RowInfo decode_row(i64 r, i64 R, const i64* __restric
         ri.u = (int)(rem - (i64)ri.t * (U + 1));
     }
     return ri;
+}
+
+__device__ __forceinline__ RowInfo decode_row(i64 r, i64 R, const i64* __restrict__ row_off,
+                                              const int* __restrict__ lx, const int* __restrict__ ly,
+                                              int N) {
+    if (N <= 0) {
+        RowInfo ri;
+        ri.n = -1; ri.t = 0; ri.u = 0; ri.T = 0; ri.U = 0; ri.off = 0;
+        return ri;
+    }
+    int lo = 0, hi = N - 1;
+    while (lo < hi) {  // last n with row_off[n] <= r (skips empty sequences)
+        int mid = (lo + hi + 1) >> 1;
+        if (row_off[mid] <= r) lo = mid; else hi = mid - 1;
+    }
+    return place_row(r, lo, R, row_off, lx, ly);
 }
 
 __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restrict__ y, i64 y_stride,

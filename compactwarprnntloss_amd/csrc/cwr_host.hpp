@@ -57,7 +57,7 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo);
 int launch_rowinfo(const Batch& b, int* rowinfo);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
-int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs);
+int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs);
 int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs);
 // d(total) / d(cost of sequence n) = p[n * stride] * scale; stride 0 broadcasts one value
 struct GradOut {

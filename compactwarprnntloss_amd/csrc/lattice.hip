@@ -403,12 +403,17 @@ int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
 __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
                                                const i64* __restrict__ pad_off, int N, i64 R,
+                                               const int2* __restrict__ rowinfo,
                                                const double2* __restrict__ lp, const double* __restrict__ alpha,
                                                const double* __restrict__ beta, float2* __restrict__ grads,
                                                float* __restrict__ costs, int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
-    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+    // the gather pass has already found the row's sequence
+    const int n = rowinfo[r].y;
+    RowInfo ri;
+    ri.n = -1;
+    if (n >= 0 && n < N) ri = place_row(r, n, R, row_off, lx, ly);
     const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
     if (pad < 0) {
         grads[r] = make_float2(0.f, 0.f);
@@ -442,11 +447,12 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
     }
 }
 
-int launch_fill(const Batch& b, const Workspace& ws, float* grads, float* costs) {
+int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs) {
     if (b.R == 0) return CWR_OK;
     unsigned blocks = (unsigned)((b.R + 255) / 256);
     hipLaunchKernelGGL(k_fill, dim3(blocks), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off, ws.pad_off, b.N,
-                       b.R, ws.lp, ws.alpha, ws.beta, reinterpret_cast<float2*>(grads), costs, b.status);
+                       b.R, reinterpret_cast<const int2*>(rowinfo), ws.lp, ws.alpha, ws.beta,
+                       reinterpret_cast<float2*>(grads), costs, b.status);
     return check_launch();
 }
 
