@@ -9,7 +9,7 @@ namespace cwr {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t pad_off, bnd_off, lp, alpha, beta, bnd_a, bnd_b, aux, total;
+    size_t pad_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
     i64 slot_cap, bnd_cap;
 };
 
@@ -30,9 +30,12 @@ static Layout layout_for(i64 N, i64 R, i64 max_u) {
     size_t at = 0;
     l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
-    l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double2));
+    l.seqmode = at; at = align_up(at + (size_t)(n + 1) * sizeof(int));
+    l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(LpCell));
     l.alpha = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
     l.beta = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
+    l.scale_a = at; at = align_up(at + ((size_t)l.slot_cap / 16 + 1) * sizeof(int));
+    l.scale_b = at; at = align_up(at + ((size_t)l.slot_cap / 16 + 1) * sizeof(int));
     l.bnd_a = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
     l.bnd_b = at; at = align_up(at + (size_t)l.bnd_cap * sizeof(double));
     l.aux = at; at = align_up(at + (size_t)r * 12);  // cwr_loss: row records (8 B) + lse (4 B) per row
@@ -48,7 +51,10 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
     char* p = static_cast<char*>(base);
     ws->pad_off = reinterpret_cast<i64*>(p + l.pad_off);
     ws->bnd_off = reinterpret_cast<i64*>(p + l.bnd_off);
-    ws->lp = reinterpret_cast<double2*>(p + l.lp);
+    ws->seqmode = reinterpret_cast<int*>(p + l.seqmode);
+    ws->lp = reinterpret_cast<LpCell*>(p + l.lp);
+    ws->scale_a = reinterpret_cast<int*>(p + l.scale_a);
+    ws->scale_b = reinterpret_cast<int*>(p + l.scale_b);
     ws->alpha = reinterpret_cast<double*>(p + l.alpha);
     ws->beta = reinterpret_cast<double*>(p + l.beta);
     ws->bnd_a = reinterpret_cast<double*>(p + l.bnd_a);
@@ -64,10 +70,13 @@ int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t
     if (N < 0 || R < 0 || max_u < 0) return CWR_ERR_SHAPE;
     Layout l = layout_for(N, R, max_u);
     switch (which) {
-        case 0: *offset = l.lp; *bytes = (size_t)l.slot_cap * sizeof(double2); return CWR_OK;
+        case 0: *offset = l.lp; *bytes = (size_t)l.slot_cap * sizeof(LpCell); return CWR_OK;
         case 1: *offset = l.alpha; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
         case 2: *offset = l.beta; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
         case 3: *offset = l.pad_off; *bytes = (size_t)(N + 1) * sizeof(i64); return CWR_OK;
+        case 4: *offset = l.seqmode; *bytes = (size_t)(N + 1) * sizeof(int); return CWR_OK;
+        case 5: *offset = l.scale_a; *bytes = ((size_t)l.slot_cap / 16 + 1) * sizeof(int); return CWR_OK;
+        case 6: *offset = l.scale_b; *bytes = ((size_t)l.slot_cap / 16 + 1) * sizeof(int); return CWR_OK;
     }
     return CWR_ERR_SHAPE;
 }
@@ -162,7 +171,7 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
         misaligned(status, 4))
         return CWR_ERR_ALIGN;
     return launch_offsets(lx, ly, N, R, 0, 0, 0, reinterpret_cast<i64*>(row_off),
-                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, status, nullptr,
+                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, nullptr, status, nullptr,
                           static_cast<hipStream_t>(stream));
 }
 
@@ -188,7 +197,7 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
-                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.bnd_off, status, costs, s);
+                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.bnd_off, ws.seqmode, status, costs, s);
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);

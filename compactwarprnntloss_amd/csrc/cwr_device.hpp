@@ -17,6 +17,12 @@ constexpr float kLn2 = 0.6931471805599453f;
 // "no path" marker of the lattice recursions.  Finite, so that marker - marker = 0 instead of NaN.
 constexpr double kNeg = -1.0e30;
 constexpr float kLpFloor = -1.0e30f;  // gathered log-probs are clamped to this (keeps -inf logits finite)
+// The scaled linear-domain walk renormalises every kPF = 16 steps to a maximum of 2^kLinTarget.
+// Inside a block a value can shrink by 2^(16*kLinMin) and grow by 2^(16*(kLinMax+1)), which must
+// stay inside the fp64 range: 800 - 16*100 = -800 > -1022 and 800 + 16*9 = 944 < 1023.
+constexpr float kLinMin = -100.0f;  // base-2 log-probs below this ...
+constexpr float kLinMax = 8.0f;     // ... or above this send the sequence to the log-domain walk
+constexpr int kLinTarget = 800;
 
 // ---------------------------------------------------------------------------------------------
 // wave64 cross-lane moves.  gfx9-family DPP controls.
@@ -195,6 +201,15 @@ __host__ __device__ __forceinline__ i64 lattice_slot(i64 t, i64 u, i64 T, i64 Up
 __host__ __device__ __forceinline__ i64 boundary_entries(i64 T, i64 Up) {
     return ((Up - 1) >> 6) * (T + kBndPad);
 }
+
+// What the gather pass leaves per lattice cell: one 16-byte store per compact row; each lattice
+// walk reads the 8-byte half of its number system.
+struct __attribute__((aligned(16))) LpCell {
+    float p_blank;  // 2^l_blank
+    float p_label;  // 2^l_label
+    float l_blank;  // log2 P(blank | t,u)
+    float l_label;  // log2 P(y[u] | t,u); 0 in the last column
+};
 
 // Which sequence owns compact row r, and where in its lattice the row sits.
 struct RowInfo {

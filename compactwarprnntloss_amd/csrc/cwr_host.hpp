@@ -37,9 +37,12 @@ struct Batch {
 struct Workspace {
     i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
-    double2* lp;    // slot_cap  gathered (blank, label) log-probabilities
-    double* alpha;  // slot_cap
+    int* seqmode;   // N+1  per sequence: 0 = walk in the scaled linear domain, 1 = in the log domain
+    LpCell* lp;     // slot_cap  gathered (blank, label) log-probabilities and probabilities
+    double* alpha;  // slot_cap  log2(alpha), or alpha * 2^scale_a[block] (see seqmode)
     double* beta;   // slot_cap
+    int* scale_a;   // slot_cap/16+1  exponent of each 16-step block of a strip's alpha walk
+    int* scale_b;   // same for beta
     double* bnd_a;  // bnd_cap   alpha values handed from one 64-label strip to the next
     double* bnd_b;  // bnd_cap   same for beta
     char* aux;      // 12 R bytes  per-row outputs of the gather pass when the caller keeps none
@@ -52,7 +55,7 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
 int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t* bytes);
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* status,
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* seqmode, int* status,
                    float* costs_or_null, hipStream_t stream);
 int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo);
 int launch_rowinfo(const Batch& b, int* rowinfo);

@@ -31,9 +31,9 @@ constexpr int kMaxFrames = 1 << 20;    // keeps a strip below the 2 GiB a buffer
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, i64 bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
-__device__ __forceinline__ double2 buf_load_d2(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    v4i v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
-    return make_double2(__hiloint2double(v.y, v.x), __hiloint2double(v.w, v.z));
+__device__ __forceinline__ float2 buf_load_f2(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    v2i v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    return make_float2(__int_as_float(v.x), __int_as_float(v.y));
 }
 __device__ __forceinline__ double buf_load_d(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     v2i v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
@@ -45,9 +45,19 @@ __device__ __forceinline__ void buf_store_d(__amdgpu_buffer_rsrc_t r, int voff, 
     v.y = __double2hiint(x);
     __builtin_amdgcn_raw_buffer_store_b64(v, r, voff, soff, 0);
 }
+__device__ __forceinline__ void buf_store_zero8(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    v2i z = {0, 0};
+    __builtin_amdgcn_raw_buffer_store_b64(z, r, voff, soff, 0);
+}
 __device__ __forceinline__ void buf_store_zero16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     v4i z = {0, 0, 0, 0};
     __builtin_amdgcn_raw_buffer_store_b128(z, r, voff, soff, 0);
+}
+__device__ __forceinline__ float buf_load_f(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ void buf_store_i32(__amdgpu_buffer_rsrc_t r, int voff, int soff, int x) {
+    __builtin_amdgcn_raw_buffer_store_b32(x, r, voff, soff, 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -60,7 +70,8 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                                                 i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                                                 i64* __restrict__ row_off, i64* __restrict__ lab_off,
                                                 i64* __restrict__ pad_off, i64* __restrict__ bnd_off,
-                                                int* __restrict__ status, float* __restrict__ costs) {
+                                                int* __restrict__ seqmode, int* __restrict__ status,
+                                                float* __restrict__ costs) {
     const int lane = threadIdx.x;
     i64 carry_r = 0, carry_l = 0, carry_p = 0, carry_b = 0;
     int flags = 0;
@@ -106,6 +117,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                 }
                 pad_off[i] = ok ? ps : -1;
                 bnd_off[i] = bs;
+                seqmode[i] = 0;
             }
             if (costs && !ok) costs[i] = __int_as_float(0x7fc00000);
         }
@@ -136,10 +148,10 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
 }
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* status, float* costs,
-                   hipStream_t stream) {
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* seqmode, int* status,
+                   float* costs, hipStream_t stream) {
     hipLaunchKernelGGL(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
-                       row_off, lab_off, pad_off, bnd_off, status, costs);
+                       row_off, lab_off, pad_off, bnd_off, seqmode, status, costs);
     return check_launch();
 }
 
@@ -148,31 +160,44 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 // ---------------------------------------------------------------------------------------------
 // Walk one strip of nl columns and T frames, Q = T+nl-1 steps; step k handles row q = k (alpha)
 // or q = Q-1-k (beta) of the strip.  With a = value of the cell, B / L its blank / label log-prob:
-//   alpha: a = lse(own, nbr);  own' = a + B(t,u);    nbr' = a + L(t,u)     -> cells (t+1,u), (t,u+1)
-//   beta : a = lse(own, nbr);  own' = a + B(t-1,u);  nbr' = a + L(t,u-1)   -> cells (t-1,u), (t,u-1)
-// i.e. every cell adds the log-prob of the transition INTO its successor, so that the only
-// operations between receiving the neighbour's value and handing one's own on are those of the
-// log-sum-exp itself (beta fetches L(t,u-1) from the lane on its left one step ahead of time).
+//   alpha: a = own (+) nbr;  own' = a (x) B(t,u);    nbr' = a (x) L(t,u)     -> cells (t+1,u), (t,u+1)
+//   beta : a = own (+) nbr;  own' = a (x) B(t-1,u);  nbr' = a (x) L(t,u-1)   -> cells (t-1,u), (t,u-1)
+// i.e. every cell applies the transition INTO its successor, so that the only operations between
+// receiving the neighbour's value and handing one's own on are those of (+) itself (beta fetches
+// L(t,u-1) from the lane on its left one step ahead of time).
+//
+// Two number systems implement ((+), (x)):
+//   linear  values are probabilities times 2^C, C an integer kept per block of kPF steps; (+) is
+//           an fp64 add and (x) an fp64 multiply, so the dependent chain of a step is
+//           DPP shift -> add -> multiply.  At the start of every block the wave takes the largest
+//           exponent among its lanes (and among the values about to come in from the previous
+//           strip), renormalises to 2^kLinTarget and records C for k_fill.  The gather pass has
+//           checked that no log-prob of the sequence can push a value out of the fp64 range
+//           within one block (kLinMin, kLinMax).
+//   log     values are base-2 logarithms in fp64, (+) is max + log2(1 + 2^-|d|) on the fp32
+//           exp2/log2 units, (x) an add.  About 3.5x slower per step; used for the sequences the
+//           gather pass marked (extreme log-probs) and for those with more strips than waves.
 //
 // Lanes that hold no cell at a step are not masked:
-//   - before its first cell a lane holds the "no path" marker (-1e30) in own and nbr'; it reads
-//     zeros from the padding (cleared below), so the marker survives (1e30 absorbs any sum);
-//   - the start cell is produced by seeding its lane's `own` (alpha[0][0] = lse(0, none) = 0,
-//     beta[T-1][U] = lse(B, none) = B);
+//   - before its first cell a lane holds "no path" (0, or -1e30 as a logarithm) in own and nbr';
+//     it reads zeros from the padding (cleared below), and "no path" survives any (x);
+//   - the start cell is produced by seeding its lane's `own`;
 //   - after its last cell a lane computes junk that no lane with a cell reads any more, and
 //     stores it into padding slots;
 //   - lanes >= nl use an offset every buffer range check rejects (loads give 0, stores vanish).
 //
 // A strip hands the values of its edge column to the next strip through a boundary stream
 // indexed by the producer's step; the receiving edge lane takes the value in as the `old` operand
-// of the DPP shift, so it lands in the lane that has no neighbour.  The stream is either a span of
-// global memory (strips walked one after the other by one wave) or a ring in LDS (strips walked
-// concurrently by one wave each, `Ring`).
+// of the DPP shift, so it lands in the lane that has no neighbour.  The stream is either a ring in
+// LDS (strips walked concurrently by one wave each) or, for the log walk of very long label
+// sequences, a span of global memory (strips walked one after the other by one wave).
 constexpr int kRing = 256;             // entries of an LDS boundary ring (a multiple of kPF)
 constexpr int kSpinLimit = 1 << 22;    // polls after which a waiting wave gives up
+constexpr int kNoExp = -(1 << 20);     // "exponent" of zero
 
 struct Ring {
-    double* slots;   // LDS, kRing entries (+ a dummy area behind them for the lanes that hold no edge)
+    double2* slots;  // LDS, kRing entries (value, exponent C of the producer) + a dummy area behind
+                     // them for the lanes that hold no edge
     int* produced;   // LDS, steps the producer has completed (INT_MAX when it is done)
     int* consumed;   // LDS, steps the consumer has completed
 };
@@ -187,54 +212,224 @@ __device__ __forceinline__ bool wait_at_least(int* counter, int need, int* statu
 }
 
 // LDS accesses of one wave are performed in program order, so a counter written after the ring
-// slots it announces needs no hardware wait; the compiler only has to keep the order.
-__device__ __forceinline__ void keep_order() { asm volatile("" ::: "memory"); }
+// slots it announces needs no hardware wait; the compiler only has to keep the order.  (A signal
+// fence emits nothing; an empty asm with a memory clobber would make the compiler drain every
+// load in flight.)
+__device__ __forceinline__ void keep_order() { __atomic_signal_fence(__ATOMIC_SEQ_CST); }
 
-template <bool BETA, bool HAS_IN, bool HAS_OUT, bool CONC>
-__device__ __forceinline__ void sweep_strip(const int T, const int nl, const bool seed, const int in_shift,
-                                            const int out_shift,
-                                            const double2* lp_strip, double* out_strip,
-                                            const double* bnd_in, double* bnd_out, const Ring rin,
-                                            const Ring rout, int* status) {
+// Waits for every load issued so far.  Placed in front of a loop whose body consumes loads issued
+// one trip earlier: the compiler derives ONE wait count per consuming instruction, the strictest
+// over all ways of reaching it, and on the way in from the initial fill the registers consumed
+// first may have been loaded last.  Without this that wait (all loads but one) would be paid on
+// every trip; with it only the loop's own distance (kPF loads) counts.
+__device__ __forceinline__ void settle_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ int exponent_of(double x) {
+    return x == 0.0 ? kNoExp : __builtin_amdgcn_frexp_exp(x);
+}
+// Maximum over the wave.  `old` = INT_MIN is the identity of max, which lets the compiler fold
+// each cross-lane move into the v_max_i32 that consumes it.
+__device__ __forceinline__ int wave_max_i32(int v) {
+    constexpr int kMin = (int)0x80000000;
+    v = max(v, dpp_i32<DPP_QUAD_XOR1>(kMin, v));
+    v = max(v, dpp_i32<DPP_QUAD_XOR2>(kMin, v));
+    v = max(v, dpp_i32<DPP_ROW_HALF_MIRROR>(kMin, v));
+    v = max(v, dpp_i32<DPP_ROW_MIRROR>(kMin, v));
+    v = max(v, dpp_i32<DPP_ROW_BCAST15, 0xA>(kMin, v));
+    v = max(v, dpp_i32<DPP_ROW_BCAST31, 0xC>(kMin, v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ double exp2_f64(float x) { return (double)fast_exp2(x); }
+
+// Both walks share one shape.  A ring of kPF registers holds the gathered records of the next
+// kPF steps; step j issues the load that refills ring[j] and prepares the NEXT step's two
+// transition terms from ring[j+1], so a ring register is dead when its refill is issued (the
+// register allocator then keeps every ring entry in place: no copies of registers with a load in
+// flight, which would make the wave wait for memory at every block) and the conversions stay off
+// the dependent chain.  The values that enter from the previous strip are prepared once per block
+// by lanes 0..kPF-1 (lane j: the value entering at step k0+j) and picked per step with a readlane.
+
+// ---- scaled linear-domain walk (strips concurrent, LDS rings) -------------------------------
+template <bool BETA, bool HAS_IN, bool HAS_OUT>
+__device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const bool seed, const int in_shift,
+                                                const int out_shift, const LpCell* lp_strip,
+                                                double* out_strip, int* scale_strip, const Ring rin,
+                                                const Ring rout, int* status) {
     const int lane = threadIdx.x & 63;
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
-    const __amdgpu_buffer_rsrc_t r_lp = make_rsrc(lp_strip, rows * nl * 16);
-    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * nl * 8);
-    const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, (HAS_IN && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
-    const __amdgpu_buffer_rsrc_t r_bo = make_rsrc(bnd_out, (HAS_OUT && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
-    const int vo_lp = lane < nl ? lane * 16 : kOob;
-    const int vo_out = lane < nl ? lane * 8 : kOob;
-    const int in_lane = BETA ? 63 : 0, out_lane = BETA ? 0 : 63;
-    const int vo_in = lane == in_lane ? 0 : kOob;
-    const int vo_bo = lane == out_lane ? 0 : kOob;
-    // LDS: the edge lane writes the ring, every other lane a private dummy slot behind it
-    double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
+    const int nblocks = (Q + kPF - 1) / kPF;
     const int p16 = nl * 16, p8 = nl * 8;
+    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
+    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
+    const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * 4);
+    const int vo_p = lane < nl ? lane * 16 : kOob;  // the two probabilities of a record
+    const int vo = lane < nl ? lane * 8 : kOob;
+    const int vo_sc = lane == 0 ? 0 : kOob;
+    constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 64 wide
+    constexpr int out_lane = BETA ? 0 : 63;
+    double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
 
-    // clear the triangle of padding slots this direction reads before a lane's first cell
+    // clear the triangle of padding records this direction reads before a lane's first cell
     for (int j = 0; j < nl - 1; ++j) {
         const int row = (BETA ? T + j : j) + kRowShift;
         const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
-        buf_store_zero16(r_lp, mine ? lane * 16 : kOob, row * p16);
+        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
     }
     __threadfence_block();
 
-    int qi = (BETA ? Q - 1 : 0) + kRowShift;  // current row
-    double2 ring[kPF];                        // log-probs of the next kPF rows
-    double ering[kPF];                        // incoming boundary values (global stream only)
+    const int row0 = (BETA ? Q - 1 : 0) + kRowShift;  // row of step 0
+    int qi = row0;                                    // row of the current step
+    int mi = BETA ? row0 - 1 : row0;                  // row that holds the current step's multipliers
+    float2 ring[kPF];                                 // (blank, label) probabilities, rows mi .. mi+dq*(kPF-1)
 #pragma unroll
-    for (int j = 0; j < kPF; ++j) {
-        ring[j] = buf_load_d2(r_lp, vo_lp, (qi + dq * j) * p16);
-        ering[j] = (HAS_IN && !CONC) ? buf_load_d(r_in, vo_in, (j + in_shift) * 8) : kNeg;
+    for (int j = 0; j < kPF; ++j) ring[j] = buf_load_f2(r_cell, vo_p, (mi + dq * j) * p16);
+    int C = kLinTarget;
+    // alpha[0][0] = 1; beta[T-1][U] = blank probability of that cell
+    double own = 0.0;
+    if (BETA) {
+        const float pb = buf_load_f(r_cell, seed ? lane * 16 : kOob, row0 * p16);
+        own = seed ? __builtin_ldexp((double)pb, kLinTarget) : 0.0;
+    } else {
+        own = seed ? __builtin_ldexp(1.0, kLinTarget) : 0.0;
     }
-    // alpha: own = 0 in the seed lane; beta: own = B of the seed lane's first cell
-    double own = seed ? (BETA ? ring[0].x : 0.0) : kNeg;
-    double pass = kNeg;
-    double nbr = kNeg;  // without an incoming stream the edge lane keeps this marker for good
+    double pass = 0.0;
+    double nbr = 0.0;  // the edge lane has no neighbour: it keeps "no path" here for good
+    // alpha applies its own cell's probabilities; beta B(t-1,u) and L(t,u-1), the latter from the
+    // lane on its left (lane 0 gets 0: nobody reads its `pass`)
+    double mul_own = (double)ring[0].x;
+    double mul_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, ring[0].y) : ring[0].y);
+    const double in_mask = lane == in_lane ? 1.0 : 0.0;
+    // beta hands on plain beta(t,u+1); the receiving edge column applies its own L(t,u), fetched
+    // one block ahead by the lanes that prepare the incoming entries
+    const int jl = lane & (kPF - 1);
+    float edge = 0.f;
+    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p16 + 63 * 16 + 4, 0);
+    settle_loads();
+    int k0 = 0;
+    for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
+        if (HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
+        if (HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+        keep_order();
+        // Renormalise.  Only lanes that still have cells count: a lane past its last cell (and a
+        // lane beyond the strip's width) carries junk of any magnitude.
+        const int first_step = BETA ? nl - 1 - lane : lane;
+        const bool alive = lane < nl && k0 - first_step < T;
+        int m = alive ? max(exponent_of(own), exponent_of(pass)) : kNoExp;
+        double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
+        int cp = 0;           // ... and the scale it was produced at
+        if (HAS_IN) {
+            const double2 en = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+            double ev = en.x;
+            if (BETA) {
+                ev *= (double)edge;
+                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p16 + 63 * 16 + 4, 0);
+            }
+            // entry k0+j feeds frame k0+j of the edge column: beyond the last frame it is junk
+            const bool ok = k0 + jl < T && ev != 0.0;
+            cp = (int)en.y;
+            e_lane = ok ? ev : 0.0;
+            if (ok) m = max(m, __builtin_amdgcn_frexp_exp(ev) + C - cp);
+        }
+        const int M = wave_max_i32(m);
+        if (M > kNoExp / 2) {
+            const int delta = kLinTarget - M;
+            own = __builtin_ldexp(own, delta);
+            pass = __builtin_ldexp(pass, delta);
+            C += delta;
+        }
+        if (HAS_IN) e_lane = __builtin_ldexp(e_lane, C - cp);
+        buf_store_i32(r_sc, vo_sc, blk * 4, C);
+        const double Cd = (double)C;
+#pragma unroll
+        for (int j = 0; j < kPF; ++j) {
+            const float2 cn = buf_load_f2(r_cell, vo_p, (mi + dq * kPF) * p16);
+            double o = own;
+            if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own);
+            nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(nbr, pass) : dpp_f64<DPP_WAVE_SHR1>(nbr, pass);
+            const double a = o + nbr;
+            own = a * mul_own;
+            pass = a * mul_pass;
+            buf_store_d(r_out, vo, qi * p8, a);
+            if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = make_double2(BETA ? a : pass, Cd);
+            const float2 nx = ring[(j + 1) % kPF];
+            mul_own = (double)nx.x;
+            mul_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, nx.y) : nx.y);
+            ring[j] = cn;
+            qi += dq;
+            mi += dq;
+            // keeps the conversions above inside this step: gathered at the top of the block they
+            // would wait for every load in flight
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        keep_order();
+        const int done = blk + 1 == nblocks ? 0x7fffffff : k0 + kPF;
+        if (HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+}
+
+// ---- log-domain walk ------------------------------------------------------------------------
+// CONC: strips concurrent, boundary values through the LDS rings; otherwise one wave walks the
+// strips in turn and the boundary values travel through a stream in global memory, which the
+// lanes that prepare the incoming entries read one block ahead.
+template <bool BETA, bool HAS_IN, bool HAS_OUT, bool CONC>
+__device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const bool seed, const int in_shift,
+                                                const int out_shift, const LpCell* lp_strip,
+                                                double* out_strip, const double* bnd_in, double* bnd_out,
+                                                const Ring rin, const Ring rout, int* status) {
+    const int lane = threadIdx.x & 63;
+    const int Q = T + nl - 1;
+    const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    int k0 = 0;  // first step of the block
+    const int p16 = nl * 16, p8 = nl * 8;
+    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
+    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
+    const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, (HAS_IN && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
+    const __amdgpu_buffer_rsrc_t r_bo = make_rsrc(bnd_out, (HAS_OUT && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
+    const int vo_l = lane < nl ? lane * 16 + 8 : kOob;  // the two logarithms of a record
+    const int vo = lane < nl ? lane * 8 : kOob;
+    constexpr int out_lane = BETA ? 0 : 63;
+    const int vo_bo = lane == out_lane ? 0 : kOob;
+    double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
+    constexpr int dq = BETA ? -1 : 1;
+
+    for (int j = 0; j < nl - 1; ++j) {
+        const int row = (BETA ? T + j : j) + kRowShift;
+        const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
+        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
+    }
+    __threadfence_block();
+
+    const int row0 = (BETA ? Q - 1 : 0) + kRowShift;
+    int qi = row0;
+    int mi = BETA ? row0 - 1 : row0;
+    float2 ring[kPF];  // (blank, label) logarithms, rows mi .. mi+dq*(kPF-1)
+#pragma unroll
+    for (int j = 0; j < kPF; ++j) ring[j] = buf_load_f2(r_cell, vo_l, (mi + dq * j) * p16);
+    // alpha: own = log 1 in the seed lane; beta: own = B of the seed lane's first cell
+    double own = kNeg;
+    if (BETA) {
+        const float lb = buf_load_f(r_cell, seed ? lane * 16 + 8 : kOob, row0 * p16);
+        own = seed ? (double)lb : kNeg;
+    } else {
+        own = seed ? 0.0 : kNeg;
+    }
+    double pass = kNeg;
+    double nbr = kNeg;
+    double add_own = (double)ring[0].x;
+    double add_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, ring[0].y) : ring[0].y);
+    const int jl = lane & (kPF - 1);
+    float edge = 0.f;      // beta: L(t,u) of the edge column's own cells, one block ahead
+    double e_next = kNeg;  // global stream: the entries of the next block
+    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p16 + 63 * 16 + 12, 0);
+    if (HAS_IN && !CONC) e_next = buf_load_d(r_in, jl * 8, in_shift * 8);
+    settle_loads();
+    int k0 = 0;
     for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
         // entries [k0+in_shift, k0+kPF+in_shift) must have been produced; the ring slots of entries
         // [k0, k0+kPF) must be free, i.e. the consumer (which reads entry i at its step
@@ -242,31 +437,25 @@ __device__ __forceinline__ void sweep_strip(const int T, const int nl, const boo
         if (CONC && HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
         if (CONC && HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
         if (CONC) keep_order();
+        double e_lane = kNeg;
+        if (HAS_IN) {
+            double ev;
+            if (CONC) {
+                ev = rin.slots[(k0 + jl + in_shift) & (kRing - 1)].x;
+            } else {
+                ev = e_next;
+                e_next = buf_load_d(r_in, jl * 8, (k0 + kPF + in_shift) * 8);
+            }
+            if (BETA) {
+                ev += (double)edge;
+                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p16 + 63 * 16 + 12, 0);
+            }
+            e_lane = k0 + jl < T ? ev : kNeg;  // beyond the last frame the entries are junk
+        }
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
-            const double2 c = ring[j];
-            // the log-probs of this lane's next cell (beta needs them now, alpha only to refill)
-            const double2 cn = buf_load_d2(r_lp, vo_lp, (qi + dq * kPF) * p16);
-            const double2 c1 = ring[(j + 1) % kPF];  // the step after this one
-            ring[j] = cn;
-            double e;
-            if (HAS_IN && CONC) {
-                e = rin.slots[(k0 + j + in_shift) & (kRing - 1)];
-            } else {
-                e = ering[j];
-                if (HAS_IN) ering[j] = buf_load_d(r_in, vo_in, (k0 + j + kPF + in_shift) * 8);
-            }
-            // what this cell adds for its two successors
-            double add_own, add_pass;
-            if (BETA) {
-                add_own = c1.x;                                   // B(t-1,u): this lane's next cell
-                add_pass = dpp_f64<DPP_WAVE_SHR1>(0.0, c1.y);     // L(t,u-1): the left lane's next cell
-                if (HAS_IN) e += c.y;                             // the stream carries plain beta(t,u+1)
-            } else {
-                add_own = c.x;
-                add_pass = c.y;
-            }
-            const double old = HAS_IN ? e : nbr;
+            const float2 cn = buf_load_f2(r_cell, vo_l, (mi + dq * kPF) * p16);
+            const double old = HAS_IN ? readlane_f64(e_lane, j) : nbr;
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(old, pass) : dpp_f64<DPP_WAVE_SHR1>(old, pass);
             const double mx = fmax(own, nbr);
             const float d = (float)(own - nbr);
@@ -274,49 +463,61 @@ __device__ __forceinline__ void sweep_strip(const int T, const int nl, const boo
             const double a = mx + l;
             own = (mx + add_own) + l;
             pass = (mx + add_pass) + l;
-            buf_store_d(r_out, vo_out, qi * p8, a);
+            buf_store_d(r_out, vo, qi * p8, a);
             if (HAS_OUT) {
-                // alpha hands on a + L(t,u) (= pass); beta hands on plain a
-                const double h = BETA ? a : pass;
-                if (CONC) ring_out[(k0 + j) & (kRing - 1)] = h;
+                const double h = BETA ? a : pass;  // alpha hands on a + L(t,u); beta plain a
+                if (CONC) ring_out[(k0 + j) & (kRing - 1)] = make_double2(h, 0.0);
                 else buf_store_d(r_bo, vo_bo, (k0 + j) * 8, h);
             }
+            const float2 nx = ring[(j + 1) % kPF];
+            add_own = (double)nx.x;
+            add_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, nx.y) : nx.y);
+            ring[j] = cn;
             qi += dq;
+            mi += dq;
+            __builtin_amdgcn_sched_barrier(0);
         }
         if (CONC) keep_order();
-        if (CONC && HAS_OUT)
-            __hip_atomic_store(rout.produced, blk + 1 == nblocks ? 0x7fffffff : k0 + kPF, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (CONC && HAS_IN)
-            __hip_atomic_store(rin.consumed, blk + 1 == nblocks ? 0x7fffffff : k0 + kPF, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_WORKGROUP);
+        const int done = blk + 1 == nblocks ? 0x7fffffff : k0 + kPF;
+        if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
 }
 
+template <bool BETA>
+__device__ __forceinline__ void lin_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
+                                             int out_shift, const LpCell* lp, double* out, int* sc, Ring rin,
+                                             Ring rout, int* status) {
+    if (has_in && has_out) sweep_strip_lin<BETA, true, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    else if (has_in) sweep_strip_lin<BETA, true, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    else if (has_out) sweep_strip_lin<BETA, false, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    else sweep_strip_lin<BETA, false, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+}
+
 template <bool BETA, bool CONC>
-__device__ __forceinline__ void sweep_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
-                                               int out_shift, const double2* lp, double* out, const double* bi, double* bo,
-                                               Ring rin, Ring rout, int* status) {
-    if (has_in && has_out) sweep_strip<BETA, true, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else if (has_in) sweep_strip<BETA, true, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else if (has_out) sweep_strip<BETA, false, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else sweep_strip<BETA, false, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+__device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
+                                             int out_shift, const LpCell* lp, double* out, const double* bi,
+                                             double* bo, Ring rin, Ring rout, int* status) {
+    if (has_in && has_out) sweep_strip_log<BETA, true, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_in) sweep_strip_log<BETA, true, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_out) sweep_strip_log<BETA, false, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else sweep_strip_log<BETA, false, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
 }
 
 // One workgroup per (sequence, direction), W waves.  A sequence of S <= W strips is walked by S
-// waves at once, each strip trailing the one that feeds it by the 64 steps the diagonal order
+// waves at once, each strip trailing the one that feeds it by the steps the diagonal order
 // demands plus one block of kPF steps of slack; the boundary values travel through LDS rings
 // guarded by two progress counters per ring.  A wave only ever waits for the wave of the strip
-// before it (values) or after it (ring space), and strip 0 waits for nobody, so the chain always
-// drains; every wait is bounded all the same.  Longer sequences (S > W) fall back to one wave
-// walking the strips in turn with the streams in global memory.
+// before it (values) or after it (ring space), and the first strip waits for nobody, so the chain
+// always drains; every wait is bounded all the same.  Longer sequences (S > W) fall back to one
+// wave walking the strips in turn, in the log domain, with the streams in global memory.
 constexpr int kMaxWaves = 8;
 
 __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
-    const i64* __restrict__ bnd_off, const double2* lp, double* alpha, double* beta, double* bnd_a,
-    double* bnd_b, int beta_only, int* status) {
-    __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
+    const i64* __restrict__ bnd_off, const int* __restrict__ seqmode, const LpCell* lp, double* alpha,
+    double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int* status) {
+    __shared__ double2 s_ring[kMaxWaves - 1][2 * kRing + 64];
     __shared__ int s_produced[kMaxWaves];
     __shared__ int s_consumed[kMaxWaves];
     const int n = blockIdx.x;
@@ -336,14 +537,15 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int S = (Up + 63) >> 6;
     const i64 full_strip = strip_rows(T, 64) * 64;
     double* out = dir ? beta : alpha;
+    int* scale = dir ? scale_b : scale_a;
     const int nl_last = Up - ((S - 1) << 6);
     Ring none;
     none.slots = nullptr; none.produced = nullptr; none.consumed = nullptr;
 
     if (S <= W) {
         // position p in the order of the walk: alpha strip p, beta strip S-1-p
+        if (w >= S) return;
         const int p = w;
-        if (p >= S) return;
         const int s = dir ? S - 1 - p : p;
         const int nl = s == S - 1 ? nl_last : 64;
         const i64 base = pad + (i64)s * full_strip;
@@ -351,15 +553,19 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         Ring rin = none, rout = none;
         if (has_in) { rin.slots = s_ring[p - 1]; rin.produced = &s_produced[p - 1]; rin.consumed = &s_consumed[p - 1]; }
         if (has_out) { rout.slots = s_ring[p]; rout.produced = &s_produced[p]; rout.consumed = &s_consumed[p]; }
-        if (dir == 0) {
-            sweep_dispatch<false, true>(has_in, has_out, T, nl, s == 0 && lane == 0, 63, 63, lp + base, out + base,
-                                        nullptr, nullptr, rin, rout, status);
+        // alpha: the feeding strip's edge lane 63 trails its first lane by 63 steps; beta: the
+        // feeding strip is s+1 and its edge lane 0 trails by its width - 1; likewise for the strip fed
+        const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
+        const int out_shift = dir ? nl - 1 : 63;
+        const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
+        const bool linear = seqmode[n] == 0;
+        if (linear) {
+            int* sc = scale + (base >> 4);
+            if (dir == 0) lin_dispatch<false>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
+            else lin_dispatch<true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
         } else {
-            // the strip that feeds strip s is s+1; its edge lane 0 trails its first lane by nl-1 steps
-            const int shift = (s + 1 == S - 1 ? nl_last : 64) - 1;
-            // ... and this strip's own edge lane 0 trails by nl-1, which is what its consumer sees
-            sweep_dispatch<true, true>(has_in, has_out, T, nl, s == S - 1 && lane == nl - 1, shift, nl - 1,
-                                       lp + base, out + base, nullptr, nullptr, rin, rout, status);
+            if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+            else log_dispatch<true, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
         }
         return;
     }
@@ -375,38 +581,66 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         // stream j runs between the strips at positions j and j+1 of the walk
         const double* bi = bnd + (i64)(p > 0 ? p - 1 : 0) * bstride;
         double* bo = bnd + (i64)p * bstride;
-        if (dir == 0) {
-            sweep_dispatch<false, false>(has_in, has_out, T, nl, s == 0 && lane == 0, 63, 63, lp + base, out + base,
-                                         bi, bo, none, none, status);
-        } else {
-            const int shift = (s + 1 == S - 1 ? nl_last : 64) - 1;
-            sweep_dispatch<true, false>(has_in, has_out, T, nl, s == S - 1 && lane == nl - 1, shift, nl - 1,
-                                        lp + base, out + base, bi, bo, none, none, status);
-        }
+        const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
+        const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
+        if (dir == 0) log_dispatch<false, false>(has_in, has_out, T, nl, seed, in_shift, 63, lp + base, out + base, bi, bo, none, none, status);
+        else log_dispatch<true, false>(has_in, has_out, T, nl, seed, in_shift, nl - 1, lp + base, out + base, bi, bo, none, none, status);
         __threadfence_block();
     }
 }
 
+// one wave per strip of the longest label sequence the call admits, up to the concurrent limit
+static int lattice_waves(const Batch& b) {
+    const i64 strips = (b.max_u + 64) / 64;
+    return (int)(strips < kMaxWaves ? (strips < 1 ? 1 : strips) : kMaxWaves);
+}
+
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
     if (b.N == 0) return CWR_OK;
-    i64 strips = (b.max_u + 64) / 64;
-    int waves = (int)(strips < 1 ? 1 : (strips > kMaxWaves ? kMaxWaves : strips));
     dim3 grid((unsigned)b.N, beta_only ? 1 : 2);
-    hipLaunchKernelGGL(k_lattice, grid, dim3(waves * 64), 0, b.stream, b.lx, b.ly, ws.pad_off, ws.bnd_off, ws.lp,
-                       ws.alpha, ws.beta, ws.bnd_a, ws.bnd_b, beta_only ? 1 : 0, b.status);
+    hipLaunchKernelGGL(k_lattice, grid, dim3(lattice_waves(b) * 64), 0, b.stream, b.lx, b.ly, ws.pad_off,
+                       ws.bnd_off, ws.seqmode, ws.lp, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, ws.bnd_a,
+                       ws.bnd_b, beta_only ? 1 : 0, b.status);
     return check_launch();
 }
 
 // ---------------------------------------------------------------------------------------------
 // per-row gradient w.r.t. the gathered log-probs, and the costs
 // ---------------------------------------------------------------------------------------------
+// Base-2 logarithm of the lattice value stored for cell (t,u): either stored as such (log walk),
+// or as value * 2^C with C recorded per block of kPF steps of the strip's walk (linear walk).
+struct LatticeView {
+    const double* v;
+    const int* scale;
+    i64 pad;
+    int T, Up;
+    bool linear, beta;
+    __device__ __forceinline__ double log2_at(int t, int u) const {
+        const i64 slot = pad + lattice_slot(t, u, T, Up);
+        const double x = v[slot];
+        if (!linear) return x;
+        const int s = u >> 6, l = u & 63;
+        const int nl = Up - (s << 6) < 64 ? Up - (s << 6) : 64;
+        const int q = t + l;
+        const int k = beta ? (T + nl - 2 - q) : q;
+        const i64 base = pad + (i64)s * strip_rows(T, 64) * 64;
+        const int C = scale[(base >> 4) + (k / kPF)];
+        // log2 x = exponent + log2(mantissa), mantissa in [0.5, 1)
+        const int ex = __builtin_amdgcn_frexp_exp(x);
+        const float mant = (float)__builtin_amdgcn_frexp_mant(x);
+        return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
+    }
+};
+
 __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
-                                               const i64* __restrict__ pad_off, int N, i64 R,
-                                               const int2* __restrict__ rowinfo,
-                                               const double2* __restrict__ lp, const double* __restrict__ alpha,
-                                               const double* __restrict__ beta, float2* __restrict__ grads,
-                                               float* __restrict__ costs, int* __restrict__ status) {
+                                               const i64* __restrict__ pad_off,
+                                               const int* __restrict__ seqmode, int N, i64 R,
+                                               const int2* __restrict__ rowinfo, const LpCell* __restrict__ lp,
+                                               const double* __restrict__ alpha, const double* __restrict__ beta,
+                                               const int* __restrict__ scale_a, const int* __restrict__ scale_b,
+                                               float2* __restrict__ grads, float* __restrict__ costs,
+                                               int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
     // the gather pass has already found the row's sequence
@@ -420,23 +654,28 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
         return;
     }
     const int T = ri.T, U = ri.U, t = ri.t, u = ri.u;
-    const i64 Up = (i64)U + 1;
-    const i64 idx = pad + lattice_slot(t, u, T, Up);
-    const double a = alpha[idx];
-    const double2 c = lp[idx];
-    const double b00 = beta[pad + lattice_slot(0, 0, T, Up)];
+    const int Up = U + 1;
+    const int S = (Up + 63) >> 6;
+    const bool linear = seqmode[ri.n] == 0 && S <= kMaxWaves;
+    LatticeView A, Bv;
+    A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear; A.beta = false;
+    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear; Bv.beta = true;
+    const double a = A.log2_at(t, u);
+    const LpCell cell = lp[pad + lattice_slot(t, u, T, Up)];
+    const float2 c = make_float2(cell.l_blank, cell.l_label);
+    const double b00 = Bv.log2_at(0, 0);
     // all values are base-2 logarithms
     float gb = 0.f, gl = 0.f;
     if (t < T - 1) {
-        gb = -fast_exp2((float)(a + beta[pad + lattice_slot(t + 1, u, T, Up)] + c.x - b00));
+        gb = -fast_exp2((float)(a + Bv.log2_at(t + 1, u) + (double)c.x - b00));
     } else if (u == U) {
-        gb = -fast_exp2((float)(a + c.x - b00));
+        gb = -fast_exp2((float)(a + (double)c.x - b00));
     }
-    if (u < U) gl = -fast_exp2((float)(a + beta[pad + lattice_slot(t, u + 1, T, Up)] + c.y - b00));
+    if (u < U) gl = -fast_exp2((float)(a + Bv.log2_at(t, u + 1) + (double)c.y - b00));
     grads[r] = make_float2(gb, gl);
     if (t == T - 1 && u == U) {
         // cwarp_cuda_rnnt_kernel.cu:353-366
-        double fa = a + c.x;
+        double fa = a + (double)c.x;
         double fb = b00;
         double ratio = fabs(fa - fb) / fabs(fmax(fa, fb));
         if (ratio > 1e-3) {
@@ -450,27 +689,32 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs) {
     if (b.R == 0) return CWR_OK;
     unsigned blocks = (unsigned)((b.R + 255) / 256);
-    hipLaunchKernelGGL(k_fill, dim3(blocks), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off, ws.pad_off, b.N,
-                       b.R, reinterpret_cast<const int2*>(rowinfo), ws.lp, ws.alpha, ws.beta,
-                       reinterpret_cast<float2*>(grads), costs, b.status);
+    hipLaunchKernelGGL(k_fill, dim3(blocks), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off, ws.pad_off,
+                       ws.seqmode, b.N, b.R, reinterpret_cast<const int2*>(rowinfo), ws.lp, ws.alpha, ws.beta,
+                       ws.scale_a, ws.scale_b, reinterpret_cast<float2*>(grads), costs, b.status);
     return check_launch();
 }
 
 __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ lx, const int* __restrict__ ly,
-                                                       const i64* __restrict__ pad_off, int N,
+                                                       const i64* __restrict__ pad_off,
+                                                       const int* __restrict__ seqmode, int N,
                                                        const double* __restrict__ beta,
+                                                       const int* __restrict__ scale_b,
                                                        float* __restrict__ costs) {
     const int n = blockIdx.x * 64 + threadIdx.x;
     if (n >= N) return;
     const i64 pad = pad_off[n];
     if (pad < 0) return;  // NaN already set by k_offsets
-    costs[n] = (float)(-beta[pad + lattice_slot(0, 0, lx[n], (i64)ly[n] + 1)] * (double)kLn2);
+    LatticeView Bv;
+    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
+    Bv.linear = seqmode[n] == 0 && ((Bv.Up + 63) >> 6) <= kMaxWaves;
+    costs[n] = (float)(-Bv.log2_at(0, 0) * (double)kLn2);
 }
 
 int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs) {
     if (b.N == 0) return CWR_OK;
     hipLaunchKernelGGL(k_cost_from_beta, dim3((unsigned)((b.N + 63) / 64)), dim3(64), 0, b.stream, b.lx,
-                       b.ly, ws.pad_off, b.N, ws.beta, costs);
+                       b.ly, ws.pad_off, ws.seqmode, b.N, ws.beta, ws.scale_b, costs);
     return check_launch();
 }
 

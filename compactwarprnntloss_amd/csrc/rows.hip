@@ -112,12 +112,21 @@ template <> struct Pack<double> {
     }
 };
 
-// What the lattice walk consumes: (blank, label) log-probabilities as base-2 logarithms in fp64,
-// floored so that -inf logits stay finite.
-__device__ __forceinline__ double2 make_lp(float xb, float xl, float lse) {
-    const double b = ((double)fmaxf(xb, kLpFloor) - (double)lse) * 1.4426950408889634;
-    const double l = ((double)fmaxf(xl, kLpFloor) - (double)lse) * 1.4426950408889634;
-    return make_double2(b, l);
+// What the lattice walk consumes, one 16-byte record per cell (see LpCell): the (blank, label)
+// log-probabilities as base-2 logarithms, floored so that -inf logits stay finite, and the same
+// two as plain probabilities for the scaled linear-domain walk.  A logarithm outside
+// [kLinMin, kLinMax] cannot be carried by that walk within one of its blocks (nor, as a
+// probability, by fp32); the sequence is then marked for the log-domain walk.
+__device__ __forceinline__ LpCell make_lp(float xb, float xl, float lse, bool has_label, int* seqmode_n) {
+    const float b = (float)(((double)fmaxf(xb, kLpFloor) - (double)lse) * 1.4426950408889634);
+    const float l = has_label ? (float)(((double)fmaxf(xl, kLpFloor) - (double)lse) * 1.4426950408889634) : 0.f;
+    if (!(b >= kLinMin && b <= kLinMax && l >= kLinMin && l <= kLinMax)) atomicOr(seqmode_n, 1);
+    LpCell c;
+    c.p_blank = fast_exp2(b);
+    c.p_label = fast_exp2(l);
+    c.l_blank = b;
+    c.l_label = l;
+    return c;
 }
 
 // position of column `col` inside a row that LPR lanes hold as K packs of VEC
@@ -220,8 +229,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ status) {
+    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     // beyond 32 values per lane the register vector would be indexed through scratch memory:
     // the two entries are then read back from the row itself (it has just been fetched)
@@ -263,7 +272,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     if (lane == 0) {
         lse_out[r] = lse;
         rowinfo[r] = make_int2(lab, ri.n);
-        if (dst >= 0) lp[dst] = make_lp(xb, lab >= 0 ? xl : lse, lse);
+        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
     }
 }
 
@@ -286,8 +295,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ status) {
+    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;   // rows per pass
     constexpr int ROWS = RP * NP;  // rows per wave
@@ -385,7 +394,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     if (mine) {
         lse_out[r] = res_lse;
         rowinfo[r] = make_int2(my_lab, ri.n);
-        if (my_dst >= 0) lp[my_dst] = make_lp(res_b, my_lab >= 0 ? res_l : res_lse, res_lse);
+        if (my_dst >= 0) lp[my_dst] = make_lp(res_b, res_l, res_lse, my_lab >= 0, seqmode + ri.n);
     }
 }
 
@@ -395,8 +404,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ status) {
+    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    int* __restrict__ seqmode, int* __restrict__ status) {
     const int lane = threadIdx.x & 63;
     const i64 r = wave_first_row(1);
     if (r >= R) return;
@@ -419,7 +428,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
-            lp[dst] = make_lp(xb, xl, lse);
+            lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
         }
         rowinfo[r] = make_int2(lab, ri.n);
     }
@@ -431,7 +440,8 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    double2* __restrict__ lp, int2* __restrict__ rowinfo, int* __restrict__ status) {
+    LpCell* __restrict__ lp, int2* __restrict__ rowinfo, int* __restrict__ seqmode,
+    int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
     const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
@@ -443,7 +453,7 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
         const T* row = x + r * (i64)V;
         const float xb = Elem<T>::to_f32(row[blank]);
         const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-        lp[dst] = make_lp(xb, xl, 0.f);
+        lp[dst] = make_lp(xb, xl, 0.f, lab >= 0, seqmode + ri.n);
     }
     rowinfo[r] = make_int2(lab, ri.n);
 }
@@ -638,13 +648,13 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
         unsigned blocks = (unsigned)((b.R + 255) / 256);
         hipLaunchKernelGGL((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
                            b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,
-                           ws.lp, ri, b.status);
+                           ws.lp, ri, ws.seqmode, b.status);
         return check_launch();
     }
     int lpr = 0, k = 0;
     if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
 #define CWR_ARGS x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,   \
-                 b.blank, ws.lp, lse, ri, b.status
+                 b.blank, ws.lp, lse, ri, ws.seqmode, b.status
         // grids are multiples of 8 workgroups, see logical_block
 #define CWR_ROW(KK)                                                                                  \
     if (lpr == 64 && k == KK) {                                                                      \
@@ -668,7 +678,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     }
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
-                       ws.pad_off, b.N, b.blank, ws.lp, lse, ri, b.status);
+                       ws.pad_off, b.N, b.blank, ws.lp, lse, ri, ws.seqmode, b.status);
     return check_launch();
 }
 

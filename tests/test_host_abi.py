@@ -50,11 +50,11 @@ def test_workspace_size_is_monotone_and_bounded():
     assert base % 256 == 0
     assert lib.cwr_workspace_bytes(32, 300000, 160) > base
     assert lib.cwr_workspace_bytes(32, 600000, 80) > base
-    # never more than 128 slots of 32 bytes per row, whatever max_u claims
+    # never more than 128 slots of 32 bytes (+ scales) per row, whatever max_u claims
     huge = lib.cwr_workspace_bytes(32, 1000, 10 ** 9)
-    assert huge < 1000 * 128 * 32 + 10 ** 6
+    assert huge < 1000 * 128 * 33 + 10 ** 6
     off, nbytes = C.c_size_t(), C.c_size_t()
-    for which in range(4):
+    for which in range(7):
         assert lib.cwr_workspace_section(32, 300000, 80, which, C.byref(off), C.byref(nbytes)) == 0
         assert off.value + nbytes.value <= base and off.value % 256 == 0
     assert lib.cwr_workspace_section(32, 300000, 80, 9, C.byref(off), C.byref(nbytes)) == 4

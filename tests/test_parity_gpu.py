@@ -277,3 +277,41 @@ def test_against_golden_fixtures(path):
         np.testing.assert_allclose(dev["costs"], z["costs"], rtol=LOSS_RTOL)
         np.testing.assert_allclose(dev["G"], z["G"], atol=GRAD_ATOL)
         np.testing.assert_allclose(dev["grad"], z["grad"], atol=GRAD_ATOL)
+
+
+# ----------------------------------------------------------------------------- number systems of the walk
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("sigma", [8.0, 25.0, 60.0])
+def test_steep_logits_linear_and_log_walks(fused, sigma):
+    """sigma 8 keeps the scaled linear-domain walk busy renormalising (about -50 bits per step);
+    25 and 60 push log-probs below the linear walk's range, so those sequences take the log walk."""
+    b = make_batch([90, 30, 150], [70, 3, 140], 200, seed=int(sigma), sigma=sigma, normalised=not fused)
+    check_case(b, fused)
+
+
+def test_mixed_batch_one_extreme_sequence():
+    """Only the sequence with extreme log-probs is marked for the log-domain walk."""
+    b = make_batch([40, 60, 35, 80], [20, 70, 5, 10], 64, seed=77, sigma=2.0)
+    off = orc.row_offsets_i64(b["lx"], b["ly"])
+    x = b["x"].clone()
+    x[off[1]:off[2]] *= 40.0
+    b["x"] = x
+    b["x_ref"] = x.to(torch.float64).numpy()
+    dev, ref = check_case(b, True)
+    assert np.all(np.isfinite(dev["costs"]))
+
+
+def test_minus_inf_logits_stay_finite_where_a_path_exists():
+    """A vocabulary entry masked with -inf that no label uses must not disturb the loss."""
+    b = make_batch([12, 7], [4, 3], 16, seed=5)
+    x = b["x"].clone()
+    x[:, 15] = -float("inf")
+    b["yp"][b["yp"] == 15] = 14
+    b["yc"][b["yc"] == 15] = 14
+    b["x"] = x
+    b["x_ref"] = x.to(torch.float64).numpy()
+    dev = run_device(b, True)
+    with np.errstate(all="ignore"):
+        ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "fused")
+    np.testing.assert_allclose(dev["costs"], ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(dev["grad"], ref["grad"], atol=GRAD_ATOL)
