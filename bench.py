@@ -86,6 +86,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0, help="seconds of CPU work for the baseline")
+    ap.add_argument("--with-pack", action="store_true",
+                    help="also time the padded -> compact pack op and its backward on the padded form of the same "
+                         "batch (reported under 'pack_op'; not part of 'value')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so that a counter run can scale "
                          "FETCH_SIZE / WRITE_SIZE against it")
@@ -184,6 +187,27 @@ def main():
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": measured_traffic("k_grad", args.config)},
     }
+
+    if args.with_pack:
+        Tm, Up = int(cfg["lx"].max()), int(cfg["ly"].max()) + 1
+        x4 = torch.zeros((N, Tm, Up, V), dtype=tdt, device=dev)
+        packed = pkg.pack_padded(x4, lx, ly, total_rows=R)
+        lib = pkg._lib.load()
+        row_off, _st = pkg.loss._offsets(lx, ly, R)
+        g4 = torch.empty_like(x4)
+        dt = pkg.loss._DTYPES[tdt]
+        stream = torch.cuda.current_stream().cuda_stream
+        pack_ms = timed(lambda: lib.cwr_pack(x4.data_ptr(), dt, N, Tm, Up, V, lx.data_ptr(), ly.data_ptr(),
+                                             row_off.data_ptr(), R, packed.data_ptr(), None, stream))
+        unpack_ms = timed(lambda: lib.cwr_unpack(packed.data_ptr(), dt, N, Tm, Up, V, lx.data_ptr(), ly.data_ptr(),
+                                                 row_off.data_ptr(), R, g4.data_ptr(), stream))
+        padded_bytes = x4.numel() * esize
+        result["pack_op"] = {
+            "padded_shape": [N, Tm, Up, V], "pack_ms": round(pack_ms, 4), "unpack_ms": round(unpack_ms, 4),
+            # pack: read + write the R valid rows; unpack: read them, write every padded row
+            "pack_GBs": round(2 * R * V * esize / (pack_ms * 1e-3) / 1e9, 1),
+            "unpack_GBs": round((R * V * esize + padded_bytes) / (unpack_ms * 1e-3) / 1e9, 1)}
+        del x4, g4, packed
 
     if not args.no_cpu:
         g_all = pkg.rnnt_backward(xd, lx, y, ly, 0, st, go, out=out)

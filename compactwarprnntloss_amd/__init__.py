@@ -3,7 +3,9 @@
 `transducer_loss` keeps the entry point of CompactWarpRNNTLoss (cwarp_rnnt/__init__.py:32-73);
 the work is done by hand-written HIP kernels behind the C ABI of include/cwarp_rnnt_hip.h.
 """
-from .loss import ForwardState, rnnt_backward, rnnt_forward, transducer_loss  # noqa: F401
+from .loss import (ForwardState, lattice_state, pack_padded, rnnt_backward, rnnt_forward,  # noqa: F401
+                   rnnt_loss, transducer_loss)
 
 __version__ = "0.1.0"
-__all__ = ["transducer_loss", "rnnt_forward", "rnnt_backward", "ForwardState", "__version__"]
+__all__ = ["transducer_loss", "rnnt_loss", "pack_padded", "lattice_state", "rnnt_forward", "rnnt_backward",
+           "ForwardState", "__version__"]

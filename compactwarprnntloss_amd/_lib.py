@@ -42,6 +42,9 @@ SIGNATURES = {
     "cwr_backward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int,
                                _p, _p, _p, _p, _p, _p, _i64, C.c_float, _p, _p]),
     "cwr_rowinfo": (C.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p]),
+    "cwr_export_lattice": (C.c_int, [_p, _p, _i64, _i64, _i64, _p, _sz, _i64, _i64, _p, _p, _p]),
+    "cwr_pack": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _p, _p]),
+    "cwr_unpack": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _p]),
 }
 
 _lib = None

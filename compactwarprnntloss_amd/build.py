@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libcwarp_rnnt_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "lattice.hip", "rows.hip"]
+SOURCES = ["api.hip", "lattice.hip", "rows.hip", "pack.hip"]
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off: hipcc would otherwise pair fp32 operations into packed
 # instructions, which have produced sporadic wrong results on the target machines.

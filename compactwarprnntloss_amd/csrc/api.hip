@@ -131,7 +131,7 @@ using namespace cwr;
 
 extern "C" {
 
-int cwr_version(void) { return 100; }
+int cwr_version(void) { return 110; }
 
 const char* cwr_strerror(int status) {
     switch (status) {
@@ -272,6 +272,50 @@ int cwr_rowinfo(const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t 
     Batch b = make_batch(nullptr, CWR_F32, R, V, lx, ly, y, y_stride, y_len, N, 0, CWR_MODE_LOGPROB, 0,
                          row_off, lab_off, nullptr, stream);
     return launch_rowinfo(b, rowinfo);
+}
+
+int cwr_export_lattice(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int64_t max_u,
+                       const void* workspace, size_t workspace_bytes_, int64_t T_pad, int64_t Up_pad,
+                       double* alphas, double* betas, void* stream) {
+    if (N < 0 || R < 0 || max_u < 0 || T_pad < 0 || Up_pad < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff || T_pad > 0x3fffffff || Up_pad > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (!workspace || (N > 0 && (!lx || !ly))) return CWR_ERR_NULL;
+    if (!alphas && !betas) return CWR_ERR_NULL;
+    if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(alphas, 8) || misaligned(betas, 8) ||
+        misaligned(workspace, 256))
+        return CWR_ERR_ALIGN;
+    Workspace ws;
+    if (!carve_workspace(const_cast<void*>(workspace), workspace_bytes_, N, R, max_u, &ws)) return CWR_ERR_SHAPE;
+    return launch_export(lx, ly, (int)N, T_pad, Up_pad, ws, alphas, betas, static_cast<hipStream_t>(stream));
+}
+
+static int repack_impl(const void* src, void* dst, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
+                       const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, int32_t* status,
+                       void* stream, bool unpack) {
+    if (dtype < CWR_F32 || dtype > CWR_F64) return CWR_ERR_DTYPE;
+    if (N < 0 || T_pad < 0 || Up_pad < 0 || V < 1 || R < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff || V > 0x3fffffff || T_pad > 0x3fffffff || Up_pad > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    const bool any_padded = N > 0 && T_pad > 0 && Up_pad > 0;
+    if (N > 0 && (!lx || !ly || !row_off)) return CWR_ERR_NULL;
+    if (any_padded && (unpack ? !dst : !src)) return CWR_ERR_NULL;
+    if (R > 0 && (unpack ? !src : !dst)) return CWR_ERR_NULL;
+    if (misaligned(src, elem_size(dtype)) || misaligned(dst, elem_size(dtype)) || misaligned(lx, 4) ||
+        misaligned(ly, 4) || misaligned(row_off, 8) || misaligned(status, 4))
+        return CWR_ERR_ALIGN;
+    return launch_repack(src, dst, elem_size(dtype), lx, ly, reinterpret_cast<const i64*>(row_off), N, T_pad, Up_pad,
+                         V, R, unpack, status, static_cast<hipStream_t>(stream));
+}
+
+int cwr_pack(const void* x_padded, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
+             const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* x_compact,
+             int32_t* status, void* stream) {
+    return repack_impl(x_padded, x_compact, dtype, N, T_pad, Up_pad, V, lx, ly, row_off, R, status, stream, false);
+}
+
+int cwr_unpack(const void* g_compact, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
+               const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* g_padded,
+               void* stream) {
+    return repack_impl(g_compact, g_padded, dtype, N, T_pad, Up_pad, V, lx, ly, row_off, R, nullptr, stream, true);
 }
 
 }  // extern "C"

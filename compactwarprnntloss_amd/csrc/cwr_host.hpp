@@ -71,6 +71,11 @@ struct GradOut {
 int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
                 const GradOut grad_costs, void* grad_x);
 
+int launch_export(const int* lx, const int* ly, int N, i64 T_pad, i64 Up_pad, const Workspace& ws,
+                  double* alphas_out, double* betas_out, hipStream_t stream);
+int launch_repack(const void* src, void* dst, size_t esize, const int* lx, const int* ly, const i64* row_off, i64 N,
+                  i64 T_pad, i64 Up_pad, i64 V, i64 R, bool unpack, int* status, hipStream_t stream);
+
 inline int check_launch() {
     return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;
 }

@@ -718,4 +718,47 @@ int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs) {
     return check_launch();
 }
 
+// ---------------------------------------------------------------------------------------------
+// export of alpha / beta as padded arrays of natural logarithms
+// ---------------------------------------------------------------------------------------------
+// What the reference hands back from its forward call (cwarp_cuda_rnnt_kernel.cu:383-384, 399-400,
+// 496): (N, T_pad, Up_pad) arrays, zero outside a sequence's own T x (U+1) lattice.
+__global__ __launch_bounds__(256) void k_export(const int* __restrict__ lx, const int* __restrict__ ly,
+                                                 const i64* __restrict__ pad_off,
+                                                 const int* __restrict__ seqmode, int N, i64 T_pad, i64 Up_pad,
+                                                 const double* __restrict__ alpha,
+                                                 const double* __restrict__ beta,
+                                                 const int* __restrict__ scale_a, const int* __restrict__ scale_b,
+                                                 double* __restrict__ alphas_out, double* __restrict__ betas_out) {
+    const i64 i = (i64)blockIdx.x * 256 + threadIdx.x;
+    const i64 per_seq = T_pad * Up_pad;
+    if (i >= (i64)N * per_seq) return;
+    const int n = (int)(i / per_seq);
+    const i64 rem = i - (i64)n * per_seq;
+    const int t = (int)(rem / Up_pad), u = (int)(rem - (i64)t * Up_pad);
+    const i64 pad = pad_off[n];
+    const int T = lx[n], Up = ly[n] + 1;
+    double a = 0.0, b = 0.0;
+    if (pad >= 0 && t < T && u < Up) {
+        LatticeView A, Bv;
+        const bool linear = seqmode[n] == 0 && ((Up + 63) >> 6) <= kMaxWaves;
+        A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear; A.beta = false;
+        Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear; Bv.beta = true;
+        if (alphas_out) a = A.log2_at(t, u) * 0.6931471805599453;
+        b = Bv.log2_at(t, u) * 0.6931471805599453;
+    }
+    if (alphas_out) alphas_out[i] = a;
+    if (betas_out) betas_out[i] = b;
+}
+
+int launch_export(const int* lx, const int* ly, int N, i64 T_pad, i64 Up_pad, const Workspace& ws,
+                  double* alphas_out, double* betas_out, hipStream_t stream) {
+    const i64 total = (i64)N * T_pad * Up_pad;
+    if (total == 0) return CWR_OK;
+    hipLaunchKernelGGL(k_export, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, lx, ly, ws.pad_off,
+                       ws.seqmode, N, T_pad, Up_pad, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, alphas_out,
+                       betas_out);
+    return check_launch();
+}
+
 }  // namespace cwr

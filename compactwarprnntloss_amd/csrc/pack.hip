@@ -1,0 +1,100 @@
+// Padded <-> compact layout conversion of (.., V) rows.
+//
+// Replaces the 4-D input branch of cwarp_rnnt/__init__.py:52-59, which hands a padded joiner
+// output (N, T, U+1, V) to the external `gather.cat`; here the rows of each sequence's own
+// T_i x (U_i+1) sub-lattice are selected, in the order of test/test.py:44-46.  k_repack moves
+// whole rows in 16-byte units (or element-sized units when rows are not 16-byte multiples): one
+// workgroup per 256 units of one PADDED row, whose (n, t, u) comes straight from the grid.
+//   pack:   compact[row_off[n] + t*(U_n+1) + u] = padded[n][t][u]      for t < T_n, u <= U_n
+//   unpack: padded[n][t][u] = the same compact row, or zeros outside the sub-lattice (this is the
+//           backward of pack: every element of the padded gradient is written, no memset pass)
+#include "cwr_device.hpp"
+#include "cwr_host.hpp"
+
+namespace cwr {
+
+template <typename U> struct Unit {
+    static __device__ __forceinline__ U zero() { return U(0); }
+    static __device__ __forceinline__ U load(const U* p) { return __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ void store(U* p, U v) { __builtin_nontemporal_store(v, p); }
+};
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+template <> struct Unit<v4i_t> {
+    static __device__ __forceinline__ v4i_t zero() { v4i_t z = {0, 0, 0, 0}; return z; }
+    static __device__ __forceinline__ v4i_t load(const v4i_t* p) { return __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ void store(v4i_t* p, v4i_t v) { __builtin_nontemporal_store(v, p); }
+};
+
+// grid: x = (label position u, block of 4 chunks of 64 units), y = frame t, z = sequence n (relative
+// to n0), so that no wave needs a 64-bit division and consecutive workgroups walk memory in order.
+template <typename U, bool UNPACK>
+__global__ __launch_bounds__(256) void k_repack(const U* __restrict__ src, U* __restrict__ dst,
+                                                 const int* __restrict__ lx, const int* __restrict__ ly,
+                                                 const i64* __restrict__ row_off, int n0, int T_pad, int Up_pad,
+                                                 i64 units_per_row, unsigned cblocks, i64 R,
+                                                 int* __restrict__ status) {
+    const int lane = threadIdx.x & 63;
+    const int n = n0 + (int)blockIdx.z;
+    const int t = (int)blockIdx.y;
+    const unsigned u = cblocks == 1 ? blockIdx.x : blockIdx.x / cblocks;
+    const unsigned cb = blockIdx.x - u * cblocks;
+    const int T = lx[n], Ul = ly[n];
+    if (status && t == 0 && blockIdx.x == 0 && threadIdx.x == 0 && (T > T_pad || Ul + 1 > Up_pad))
+        atomicOr(status, CWR_FLAG_BAD_LENGTH);  // part of this sequence lies outside the padded array
+    bool valid = T > 0 && Ul >= 0 && t < T && (int)u <= Ul;
+    i64 crow = 0;
+    if (valid) {
+        crow = row_off[n] + (i64)t * ((i64)Ul + 1) + u;
+        if (crow >= R) valid = false;  // lengths that do not add up to R: flagged by the offsets pass
+    }
+    if (!UNPACK && !valid) return;
+    const i64 unit = ((i64)cb * 4 + (threadIdx.x >> 6)) * 64 + lane;
+    if (unit >= units_per_row) return;
+    const i64 prow = ((i64)n * T_pad + t) * Up_pad + u;
+    if (UNPACK) {
+        U v = Unit<U>::zero();
+        if (valid) v = Unit<U>::load(src + crow * units_per_row + unit);
+        Unit<U>::store(dst + prow * units_per_row + unit, v);
+    } else {
+        Unit<U>::store(dst + crow * units_per_row + unit, Unit<U>::load(src + prow * units_per_row + unit));
+    }
+}
+
+template <typename U>
+static int repack_as(const void* src, void* dst, const int* lx, const int* ly, const i64* row_off, i64 N, i64 T_pad,
+                     i64 Up_pad, i64 units_per_row, i64 R, bool unpack, int* status, hipStream_t stream) {
+    if (N == 0 || T_pad == 0 || Up_pad == 0) return CWR_OK;
+    const i64 cblocks = (units_per_row + 255) / 256;
+    if (T_pad > 65535 || Up_pad * cblocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
+    for (i64 n0 = 0; n0 < N; n0 += 65535) {
+        const i64 nz = N - n0 < 65535 ? N - n0 : 65535;
+        dim3 grid((unsigned)(Up_pad * cblocks), (unsigned)T_pad, (unsigned)nz);
+        if (unpack)
+            hipLaunchKernelGGL((k_repack<U, true>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
+                               static_cast<U*>(dst), lx, ly, row_off, (int)n0, (int)T_pad, (int)Up_pad,
+                               units_per_row, (unsigned)cblocks, R, status);
+        else
+            hipLaunchKernelGGL((k_repack<U, false>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
+                               static_cast<U*>(dst), lx, ly, row_off, (int)n0, (int)T_pad, (int)Up_pad,
+                               units_per_row, (unsigned)cblocks, R, status);
+        int rc = check_launch();
+        if (rc != CWR_OK) return rc;
+    }
+    return CWR_OK;
+}
+
+int launch_repack(const void* src, void* dst, size_t esize, const int* lx, const int* ly, const i64* row_off, i64 N,
+                  i64 T_pad, i64 Up_pad, i64 V, i64 R, bool unpack, int* status, hipStream_t stream) {
+    const size_t row_bytes = (size_t)V * esize;
+    const bool wide = row_bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    if (wide) return repack_as<v4i_t>(src, dst, lx, ly, row_off, N, T_pad, Up_pad, (i64)(row_bytes / 16), R, unpack, status, stream);
+    switch (esize) {
+        case 2: return repack_as<unsigned short>(src, dst, lx, ly, row_off, N, T_pad, Up_pad, V, R, unpack, status, stream);
+        case 4: return repack_as<unsigned int>(src, dst, lx, ly, row_off, N, T_pad, Up_pad, V, R, unpack, status, stream);
+        case 8: return repack_as<unsigned long long>(src, dst, lx, ly, row_off, N, T_pad, Up_pad, V, R, unpack, status, stream);
+    }
+    return CWR_ERR_DTYPE;
+}
+
+}  // namespace cwr

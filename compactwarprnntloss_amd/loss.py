@@ -9,6 +9,8 @@ additive keyword arguments:
   fused_log_softmax  False (default): x holds log-probabilities and the gradient is the
                      reference's sparse one.  True: x holds raw logits, log-softmax over V is
                      fused into the gather pass, the gradient w.r.t. the logits is dense.
+  x of 4 dims        a padded (N, T, U+1, V) tensor is packed first (pack_padded), as the
+                     reference does through gather.cat (cwarp_rnnt/__init__.py:52-59)
   max_u              host-known upper bound of max(ly) for concatenated 1-D labels
   validate           read the device status word back (one synchronisation) and raise on
                      data-dependent problems.  Off by default: the hot path never synchronises.
@@ -132,6 +134,98 @@ def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torc
     return out
 
 
+def lattice_state(st: ForwardState, lx, ly, t_pad: int, up_pad: int, with_alpha: bool = True):
+    """Binding of cwr_export_lattice: (alphas, betas) as (N, t_pad, up_pad) float64 natural logs, zero
+    outside each sequence's lattice, from the workspace a forward call left in `st` (the reference
+    returns both from its forward, cwarp_cuda_rnnt_kernel.cu:383-384,496).  After a loss-only call
+    only beta exists: pass with_alpha=False."""
+    if st.workspace is None:
+        raise RuntimeError("the forward state holds no workspace any more")
+    lib = _lib.load()
+    dev = lx.device
+    alphas = torch.empty((st.N, t_pad, up_pad), dtype=torch.float64, device=dev) if with_alpha else None
+    betas = torch.empty((st.N, t_pad, up_pad), dtype=torch.float64, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.cwr_export_lattice(lx.data_ptr(), ly.data_ptr(), st.N, st.R, st.max_u, st.workspace.data_ptr(),
+                                    st.workspace.numel(), int(t_pad), int(up_pad),
+                                    alphas.data_ptr() if with_alpha else None, betas.data_ptr(), _stream_ptr(dev))
+        _lib.check(rc, "cwr_export_lattice")
+    return alphas, betas
+
+
+def _offsets(lx, ly, total_rows: int):
+    """Binding of cwr_offsets: (row_off (N+1) int64, status 4 x int32) on the device."""
+    lib = _lib.load()
+    dev = lx.device
+    N = lx.numel()
+    meta = torch.empty(2 * (N + 1) + 2, dtype=torch.int64, device=dev)
+    status = meta[2 * (N + 1):].view(torch.int32)
+    with torch.cuda.device(dev):
+        rc = lib.cwr_offsets(lx.data_ptr(), ly.data_ptr(), N, int(total_rows), meta.data_ptr(),
+                             meta[N + 1:].data_ptr(), status.data_ptr(), _stream_ptr(dev))
+        _lib.check(rc, "cwr_offsets")
+    return meta[: N + 1], status
+
+
+class _Pack(torch.autograd.Function):
+    """Padded (N, T, U+1, V) -> compact (R, V) and its backward (cwr_pack / cwr_unpack)."""
+
+    @staticmethod
+    def forward(ctx: Any, x4, lx, ly, total_rows):
+        lib = _lib.load()
+        N, T, Up, V = x4.shape
+        row_off, status = _offsets(lx, ly, total_rows)
+        out = torch.empty((total_rows, V), dtype=x4.dtype, device=x4.device)
+        with torch.cuda.device(x4.device):
+            rc = lib.cwr_pack(x4.data_ptr(), _DTYPES[x4.dtype], N, T, Up, V, lx.data_ptr(), ly.data_ptr(),
+                              row_off.data_ptr(), total_rows, out.data_ptr(), status.data_ptr(),
+                              _stream_ptr(x4.device))
+            _lib.check(rc, "cwr_pack")
+        ctx.save_for_backward(lx, ly, row_off)
+        ctx.shape = (N, T, Up, V)
+        ctx.status = status
+        return out
+
+    @staticmethod
+    def backward(ctx: Any, g):
+        lx, ly, row_off = ctx.saved_tensors
+        N, T, Up, V = ctx.shape
+        lib = _lib.load()
+        g = g.contiguous()
+        out = torch.empty((N, T, Up, V), dtype=g.dtype, device=g.device)
+        with torch.cuda.device(g.device):
+            rc = lib.cwr_unpack(g.data_ptr(), _DTYPES[g.dtype], N, T, Up, V, lx.data_ptr(), ly.data_ptr(),
+                                row_off.data_ptr(), g.size(0), out.data_ptr(), _stream_ptr(g.device))
+            _lib.check(rc, "cwr_unpack")
+        return out, None, None, None
+
+
+def pack_padded(x: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
+                total_rows: Optional[int] = None) -> torch.Tensor:
+    """Compact layout (sum_i T_i*(U_i+1), V) of a padded joiner output (N, T, U+1, V): for every
+    sequence the rows of its own T_i x (U_i+1) sub-lattice, t-major (test/test.py:44-46).
+    Differentiable.  Takes the place of `gather.cat` in cwarp_rnnt/__init__.py:52-59, which keeps the
+    FIRST T_i*(U_i+1) rows of the flattened sequence instead and therefore only agrees with the
+    compact layout when every U_i equals the padded width.
+
+    total_rows: sum_i T_i*(U_i+1) if the caller knows it; otherwise it is computed on the device and
+    read back (one synchronisation)."""
+    if x.dim() != 4:
+        raise RuntimeError("x must be (N, T, U+1, V)")
+    if not x.is_cuda or not x.is_contiguous():
+        raise RuntimeError("x must be a contiguous CUDA tensor")
+    if x.dtype not in _DTYPES:
+        raise RuntimeError(f"unsupported dtype {x.dtype}")
+    for name, t in (("lx", lx), ("ly", ly)):
+        if not t.is_cuda or t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous CUDA int32 tensor")
+    if lx.numel() != x.size(0) or ly.numel() != x.size(0):
+        raise RuntimeError("lx, ly must hold one entry per sequence")
+    if total_rows is None:
+        total_rows = int((lx.long() * (ly.long() + 1)).sum().item())
+    return _Pack.apply(x, lx, ly, int(total_rows))
+
+
 def _raise_on_flags(st: ForwardState):
     flags = int(st.status[0].item())
     hard = flags & ~_lib.FLAG_FB_MISMATCH
@@ -146,13 +240,15 @@ class _TransLoss(torch.autograd.Function):
     instead of materialising an expanded per-sequence tensor."""
 
     @staticmethod
-    def forward(ctx: Any, xs, lx, ys, ly, blank, fused, max_u, validate, reduction):
+    def forward(ctx: Any, xs, lx, ys, ly, blank, fused, max_u, validate, reduction, fastemit_lambda=0.0):
         need_grad = xs.requires_grad
         costs, st = rnnt_forward(xs, lx, ys, ly, blank, fused, max_u, with_grad=need_grad)
         if validate:
             _raise_on_flags(st)
         if need_grad:
             st.workspace = None  # alpha / beta are not needed again
+            if fastemit_lambda:
+                st.grads[:, 1] *= 1.0 + fastemit_lambda
             ctx.state = st
             ctx.blank = blank
             ctx.reduction = reduction
@@ -170,7 +266,7 @@ class _TransLoss(torch.autograd.Function):
         xs, lx, ys, ly = ctx.saved_tensors
         scale = 1.0 / ctx.state.N if ctx.reduction == "mean" else 1.0
         grad_input = rnnt_backward(xs, lx, ys, ly, ctx.blank, ctx.state, grad_outputs, scale=scale)
-        return grad_input, None, None, None, None, None, None, None, None
+        return grad_input, None, None, None, None, None, None, None, None, None
 
 
 def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torch.Tensor, blank: int = 0,
@@ -194,6 +290,12 @@ def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torc
     assert lx.size(0) == ly.size(0)
     assert blank >= 0 and blank < x.size(-1)
     del gather  # always on, as in the reference
+    if x.dim() == 4:
+        # cwarp_rnnt/__init__.py:52-59
+        import warnings
+        warnings.warn("transducer_loss: 4-D input is packed into the compact layout first; pass compact "
+                      "(sum_i T_i*(U_i+1), V) input to skip that copy", stacklevel=2)
+        x = pack_padded(x if x.is_contiguous() else x.contiguous(), lx, ly)
     # x: (STU, V)
     assert x.dim() == 2, "input must be compact: (sum_i T_i*(U_i+1), V)"
 
@@ -201,3 +303,42 @@ def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torc
         raise ValueError
     return _TransLoss.apply(x, lx, y, ly, blank, bool(fused_log_softmax), max_u, bool(validate),
                             reduction if reduction in ("mean", "sum") else "none")
+
+
+def rnnt_loss(log_probs: torch.Tensor, labels: torch.Tensor, frames_lengths: torch.Tensor,
+              labels_lengths: torch.Tensor, average_frames: bool = False, reduction: Optional[str] = None,
+              blank: int = 0, gather: bool = False, fastemit_lambda: float = 0.0,
+              compact: bool = False) -> torch.Tensor:
+    """Front end with the call signature of `warp_rnnt.rnnt_loss`, the sibling API the reference's own
+    test drives next to `transducer_loss` (test/test.py:4,67), on top of the same kernels.
+
+    log_probs       (N, T, U+1, V) log-probabilities, or with compact=True (sum_i T_i*(U_i+1), V)
+    labels          (N, U) padded, or with compact=True (sum_i U_i,) concatenated (padded accepted)
+    average_frames  divide every sequence's loss by its frame count
+    reduction       None / "none", "mean", "sum"
+    gather          accepted; the gather of the blank and label columns is always on here
+    fastemit_lambda scales the gradient of every label emission by (1 + lambda) and leaves the loss
+                    value alone (FastEmit as a gradient re-weighting)
+    """
+    assert reduction in (None, "none", "mean", "sum")
+    del gather
+    if labels.dtype != torch.int32:
+        labels = labels.int()
+    lx = frames_lengths if frames_lengths.dtype == torch.int32 else frames_lengths.int()
+    ly = labels_lengths if labels_lengths.dtype == torch.int32 else labels_lengths.int()
+    x = log_probs
+    if not compact:
+        if x.dim() != 4:
+            raise RuntimeError("log_probs must be (N, T, U+1, V) unless compact=True")
+        x = pack_padded(x if x.is_contiguous() else x.contiguous(), lx, ly)
+    elif x.dim() != 2:
+        raise RuntimeError("compact log_probs must be (sum_i T_i*(U_i+1), V)")
+    costs = _TransLoss.apply(x, lx, labels.contiguous(), ly, int(blank), False, None, False, "none",
+                             float(fastemit_lambda))
+    if average_frames:
+        costs = costs / lx.to(costs.dtype)
+    if reduction == "mean":
+        return costs.mean()
+    if reduction == "sum":
+        return costs.sum()
+    return costs

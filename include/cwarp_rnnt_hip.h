@@ -163,6 +163,33 @@ int cwr_rowinfo(const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t 
                 int64_t N, int64_t R, int64_t V, const int64_t* row_off, const int64_t* lab_off,
                 int32_t* rowinfo, void* stream);
 
+/* alpha and beta of the last cwr_forward (beta only after cwr_loss: pass alphas = NULL), copied
+ * out of its workspace as padded (N, T_pad, Up_pad) fp64 arrays of NATURAL logarithms, zero
+ * outside each sequence's own T x (U+1) lattice -- what the reference returns from its forward
+ * call (cwarp_cuda_rnnt_kernel.cu:383-384, 399-400, 496).  lx, ly, N, R, max_u, workspace as in
+ * that call; cells with t >= T_pad or u >= Up_pad are not exported.  Either output may be NULL. */
+int cwr_export_lattice(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int64_t max_u,
+                       const void* workspace, size_t workspace_bytes, int64_t T_pad, int64_t Up_pad,
+                       double* alphas, double* betas, void* stream);
+
+/* Padded -> compact rows.  Replaces the 4-D input branch cwarp_rnnt/__init__.py:52-59 (which
+ * calls the external gather.cat on the flattened tensor): for every sequence n the rows of its own
+ * sub-lattice, x_compact[row_off[n] + t*(ly[n]+1) + u, :] = x_padded[n, t, u, :] for t < lx[n],
+ * u <= ly[n] (the compact order of test/test.py:44-46).
+ *   x_padded (N, T_pad, Up_pad, V) contiguous;  x_compact (R, V);  row_off from cwr_offsets
+ *   status   optional 4 x int32 already initialised by cwr_offsets: CWR_FLAG_BAD_LENGTH is added
+ *            when a sequence does not fit (lx[n] > T_pad or ly[n]+1 > Up_pad); its rows beyond the
+ *            padded array are left untouched. */
+int cwr_pack(const void* x_padded, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
+             const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* x_compact,
+             int32_t* status, void* stream);
+
+/* Backward of cwr_pack: g_padded[n, t, u, :] = g_compact[row, :] inside the sub-lattice and 0
+ * elsewhere; every element of g_padded is written. */
+int cwr_unpack(const void* g_compact, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
+               const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* g_padded,
+               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,7 +26,8 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = declared_functions()
     assert {"cwr_forward", "cwr_loss", "cwr_backward", "cwr_offsets", "cwr_rowinfo", "cwr_version",
-            "cwr_strerror", "cwr_workspace_bytes", "cwr_workspace_section", "cwr_lattice_slot"} <= set(names)
+            "cwr_strerror", "cwr_workspace_bytes", "cwr_workspace_section", "cwr_lattice_slot",
+            "cwr_export_lattice", "cwr_pack", "cwr_unpack"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
     assert set(_lib.SIGNATURES) == set(names)
@@ -128,6 +129,14 @@ def test_invalid_calls_are_rejected_on_the_host():
     assert lib.cwr_backward(p(1), 0, 10, 8, None, None, None, 3, 6, 2, 0, 1, None, None, p(1), p(2), p(3),
                             p(4), 2, 1.0, p(5), None) == 4          # grad_stride is 0 or 1
     assert lib.cwr_rowinfo(p(1), p(2), p(3), 3, 6, 2, 10, 8, p(4), p(5), None, None) == 1
+    assert lib.cwr_pack(None, 0, 2, 3, 4, 8, p(1), p(2), p(3), 10, p(4), None, None) == 1   # no padded input
+    assert lib.cwr_pack(p(1), 9, 2, 3, 4, 8, p(1), p(2), p(3), 10, p(4), None, None) == 2
+    assert lib.cwr_pack(p(1), 0, 2, -3, 4, 8, p(1), p(2), p(3), 10, p(4), None, None) == 4
+    assert lib.cwr_unpack(p(1), 0, 2, 3, 4, 8, p(1), p(2), p(3), 10, None, None) == 1        # no padded output
+    assert lib.cwr_unpack(p(1) + 2, 0, 2, 3, 4, 8, p(1), p(2), p(3), 10, p(4), None) == 6
+    assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, None, 1 << 30, 4, 4, p(3), p(4), None) == 1
+    assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, p(5), 16, 4, 4, p(3), p(4), None) == 4  # workspace too small
+    assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, p(5), 1 << 30, 4, 4, None, None, None) == 1
     # R == 0 is a valid (empty) call and launches nothing that touches memory
     assert lib.cwr_backward(None, 0, 0, 8, None, None, None, 0, 0, 0, 0, 0, None, None, None, None, None,
                             None, 1, 1.0, None, None) == 0
@@ -150,7 +159,9 @@ def test_entry_point_asserts_match_the_reference():
     with pytest.raises(AssertionError):
         cwarp_rnnt.transducer_loss(x, lx, torch.zeros((2, 2), dtype=torch.int32), ly)  # y.size(0) == N
     with pytest.raises(AssertionError):
-        cwarp_rnnt.transducer_loss(x.view(1, 2, 3, 4), lx, y, ly)  # compact 2-D input only
+        cwarp_rnnt.transducer_loss(x.view(2, 3, 4), lx, y, ly)    # compact 2-D (or padded 4-D) input only
+    with pytest.warns(UserWarning), pytest.raises(RuntimeError, match="CUDA"):
+        cwarp_rnnt.transducer_loss(x.view(1, 2, 3, 4), lx, y, ly)  # 4-D input is packed: GPU only
     with pytest.raises(RuntimeError, match="CUDA"):
         cwarp_rnnt.transducer_loss(x, lx, y, ly)                  # CPU tensors are refused, no fallback
     assert cwarp_rnnt.__version__
