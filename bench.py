@@ -49,17 +49,19 @@ def measured_traffic(kernel: str, config: int):
 
 
 def cpu_baseline(cfg, x_cpu, budget_s, dev_out):
-    """Time the NumPy oracle on the first sequences of the batch (at least one, then as many as fit
-    the budget) and compare the device results on those sequences."""
+    """Time the NumPy oracle on the sequences of the batch, one after the other, for about half the
+    budget at least (going round the batch again if it is done sooner) and never beyond the budget;
+    the first time round, compare the device results on those sequences."""
+    import torch
     from oracle import rnnt_oracle as orc
     off = orc.row_offsets_i64(cfg["lx"], cfg["ly"])
     esize = x_cpu.element_size()
     t_used, n_done, bytes_done = 0.0, 0, 0
     loss_rel, grad_abs = 0.0, 0.0
     N = cfg["N"]
-    while n_done < N:
-        n = n_done
-        xs = x_cpu[off[n]:off[n + 1]].to(dtype=__import__("torch").float64).numpy()
+    while True:
+        n = n_done % N
+        xs = x_cpu[off[n]:off[n + 1]].to(dtype=torch.float64).numpy()
         lab = cfg["y_padded"][n:n + 1]
         t0 = time.perf_counter()
         ref = orc.loss_and_grad(xs, cfg["lx"][n:n + 1], lab, cfg["ly"][n:n + 1], 0, "fused",
@@ -68,14 +70,16 @@ def cpu_baseline(cfg, x_cpu, budget_s, dev_out):
         t_used += dt
         n_done += 1
         bytes_done += xs.shape[0] * cfg["V"] * 3 * esize
-        loss_rel = max(loss_rel, abs(dev_out["costs"][n] - ref["costs"][0]) / abs(ref["costs"][0]))
-        grad_abs = max(grad_abs, float(np.abs(dev_out["grad"](off[n], off[n + 1]) - ref["grad"]).max()))
-        if t_used + dt > budget_s:
+        if n_done <= N:
+            loss_rel = max(loss_rel, abs(dev_out["costs"][n] - ref["costs"][0]) / abs(ref["costs"][0]))
+            grad_abs = max(grad_abs, float(np.abs(dev_out["grad"](off[n], off[n + 1]) - ref["grad"]).max()))
+        if t_used + dt > budget_s or (n_done >= N and n_done % N == 0 and t_used >= 0.5 * budget_s):
             break
+    checked = min(n_done, N)
     return dict(value=bytes_done / t_used / 1e9, unit="GB/s", cores=1, kind="port",
-                sample=f"float64 NumPy oracle, first {n_done} of {N} sequences of the same batch, "
-                       f"{t_used:.1f} s",
-                ), dict(loss_rel_err=loss_rel, grad_abs_err=grad_abs, sequences_checked=n_done)
+                sample=f"float64 NumPy oracle, {n_done} sequence passes over the {N} sequences of the same "
+                       f"batch ({n_done / N:.1f} batches), {t_used:.1f} s",
+                ), dict(loss_rel_err=loss_rel, grad_abs_err=grad_abs, sequences_checked=checked)
 
 
 def main():
