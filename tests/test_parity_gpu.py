@@ -315,3 +315,78 @@ def test_minus_inf_logits_stay_finite_where_a_path_exists():
         ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "fused")
     np.testing.assert_allclose(dev["costs"], ref["costs"], rtol=LOSS_RTOL)
     np.testing.assert_allclose(dev["grad"], ref["grad"], atol=GRAD_ATOL)
+
+
+# ----------------------------------------------------------------------------- full benchmark sizes
+def _full_config(idx):
+    cfg = orc.make_config(idx)
+    tdt = torch.float16 if cfg["dtype"] == "f16" else torch.float32
+    g = torch.Generator(device="cpu").manual_seed(1000 + idx)
+    x = (torch.randn((cfg["R"], cfg["V"]), generator=g, dtype=torch.float32) * cfg["sigma"]).to(tdt)
+    return cfg, x
+
+
+@pytest.mark.parametrize("idx", [2, 3, 4, 5])
+def test_full_size_configs_size_independent_properties(idx):
+    """At the benchmark's own sizes: what must hold whatever the size.  Every frame leaves its
+    lattice row by exactly one blank and every label is emitted exactly once (so the sparse
+    gradients of a sequence sum to -T and -U), a dense fused gradient row sums to zero, the
+    gradient is linear in the incoming one, and the gradient and loss-only passes agree."""
+    pkg = _pkg()
+    cfg, x = _full_config(idx)
+    dev = torch.device("cuda:0")
+    xs = x.to(dev)
+    lx, ly = torch.from_numpy(cfg["lx"]).to(dev), torch.from_numpy(cfg["ly"]).to(dev)
+    ys = torch.from_numpy(cfg["y_padded"]).to(dev)
+    N = cfg["N"]
+    costs, st = pkg.rnnt_forward(xs, lx, ys, ly, 0, True)
+    costs_only, _ = pkg.rnnt_forward(xs, lx, ys, ly, 0, True, with_grad=False)
+    assert int(st.status[0].item()) == 0
+    assert torch.isfinite(costs).all() and (costs > 0).all()
+    torch.testing.assert_close(costs_only, costs, rtol=1e-6, atol=0)
+    rows = (lx.long() * (ly.long() + 1))
+    assert int(rows.sum().item()) == cfg["R"] and int(st.row_off[-1].item()) == cfg["R"]
+    seq = torch.repeat_interleave(torch.arange(N, device=dev), rows)
+    assert torch.equal(st.rowinfo[:, 1].long(), seq)
+    occ = torch.zeros((N, 2), dtype=torch.float64, device=dev).index_add_(0, seq, -st.grads.double())
+    torch.testing.assert_close(occ[:, 0], lx.double(), rtol=2e-5, atol=1e-3)
+    torch.testing.assert_close(occ[:, 1], ly.double(), rtol=2e-5, atol=1e-3)
+    w = torch.rand(N, device=dev) + 0.5
+    g1 = pkg.rnnt_backward(xs, lx, ys, ly, 0, st, w)
+    row_sum = g1.float().sum(dim=1).abs().max().item()
+    assert row_sum < (2e-5 if idx != 3 else 2e-2)      # fp16 storage rounds each of the 4096 entries
+    g2 = pkg.rnnt_backward(xs, lx, ys, ly, 0, st, w, scale=2.0)
+    # a power-of-two factor commutes with rounding (up to flushed denormals, and fp16 overflow aside)
+    torch.testing.assert_close(g2.float(), 2 * g1.float(), rtol=1e-6 if idx != 3 else 2e-3,
+                               atol=1e-30 if idx != 3 else 2e-7)   # fp16 subnormals step by 6e-8
+    del g2
+    # the blank and label columns carry the whole of the sparse gradient's mass
+    lab = st.rowinfo[:, 0].long()
+    wrow = w[seq].double()
+    pb = torch.exp(xs[:, 0].double() - st.lse.double())
+    gamma = -(st.grads.double().sum(dim=1))
+    torch.testing.assert_close(g1[:, 0].double(), wrow * (pb * gamma + st.grads[:, 0].double()),
+                               rtol=2e-3 if idx == 3 else 1e-5, atol=1e-6)
+    has = lab >= 0
+    pl = torch.exp(xs[has, lab[has]].double() - st.lse[has].double())
+    torch.testing.assert_close(g1[has, lab[has]].double(), wrow[has] * (pl * gamma[has] + st.grads[has, 1].double()),
+                               rtol=2e-3 if idx == 3 else 1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("idx", [2, 4])
+def test_full_size_configs_against_oracle(idx):
+    """Configs whose float64 oracle run takes a few seconds: direct parity at full size."""
+    pkg = _pkg()
+    cfg, x = _full_config(idx)
+    dev = torch.device("cuda:0")
+    xs = x.to(dev)
+    lx, ly = torch.from_numpy(cfg["lx"]).to(dev), torch.from_numpy(cfg["ly"]).to(dev)
+    ys = torch.from_numpy(cfg["y_padded"]).to(dev)
+    costs, st = pkg.rnnt_forward(xs, lx, ys, ly, 0, True)
+    go = np.full(cfg["N"], 1.0 / cfg["N"])
+    g = pkg.rnnt_backward(xs, lx, ys, ly, 0, st, torch.from_numpy(go).to(dev))
+    ref = orc.loss_and_grad(x.double().numpy(), cfg["lx"], cfg["y_padded"], cfg["ly"], 0, "fused", grad_out=go)
+    assert int(st.status[0].item()) == 0
+    np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
+    assert float(np.abs(g.cpu().numpy() - ref["grad"]).max()) <= GRAD_ATOL
