@@ -9,7 +9,7 @@ namespace cwr {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t pad_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
+    size_t pad_off, slot_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
     i64 slot_cap, bnd_cap;
 };
 
@@ -29,6 +29,7 @@ static Layout layout_for(i64 N, i64 R, i64 max_u) {
     l.bnd_cap = r / 64 + (bnd_by_strips < bnd_by_rows ? bnd_by_strips : bnd_by_rows) + 1;
     size_t at = 0;
     l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
+    l.slot_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.seqmode = at; at = align_up(at + (size_t)(n + 1) * sizeof(int));
     l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(LpCell));
@@ -50,6 +51,7 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
     if (bytes < l.total) return false;
     char* p = static_cast<char*>(base);
     ws->pad_off = reinterpret_cast<i64*>(p + l.pad_off);
+    ws->slot_off = reinterpret_cast<i64*>(p + l.slot_off);
     ws->bnd_off = reinterpret_cast<i64*>(p + l.bnd_off);
     ws->seqmode = reinterpret_cast<int*>(p + l.seqmode);
     ws->lp = reinterpret_cast<LpCell*>(p + l.lp);
@@ -171,7 +173,7 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
         misaligned(status, 4))
         return CWR_ERR_ALIGN;
     return launch_offsets(lx, ly, N, R, 0, 0, 0, reinterpret_cast<i64*>(row_off),
-                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, nullptr, status, nullptr,
+                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, nullptr, nullptr, status, nullptr,
                           static_cast<hipStream_t>(stream));
 }
 
@@ -197,11 +199,11 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
-                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.bnd_off, ws.seqmode, status, costs, s);
+                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.slot_off, ws.bnd_off, ws.seqmode, status, costs, s);
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
-    rc = launch_gather(b, ws, lse, rowinfo);
+    rc = launch_gather(b, ws, lse, rowinfo, with_grad ? grads : nullptr);
     if (rc != CWR_OK) return rc;
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;

@@ -36,6 +36,7 @@ struct Batch {
 // lattice_slot(); all values are base-2 logarithms.
 struct Workspace {
     i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
+    i64* slot_off;  // N+1  the same running sum without the -1 marks (monotone: searchable)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
     int* seqmode;   // N+1  per sequence: 0 = walk in the scaled linear domain, 1 = in the log domain
     LpCell* lp;     // slot_cap  gathered (blank, label) log-probabilities and probabilities
@@ -55,9 +56,10 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
 int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t* bytes);
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* seqmode, int* status,
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode, int* status,
                    float* costs_or_null, hipStream_t stream);
-int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo);
+// grads (may be null): rows of skipped sequences get a zero record there
+int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads);
 int launch_rowinfo(const Batch& b, int* rowinfo);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs);

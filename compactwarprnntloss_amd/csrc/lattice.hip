@@ -69,9 +69,9 @@ __device__ __forceinline__ void buf_store_i32(__amdgpu_buffer_rsrc_t r, int voff
 __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, const int* __restrict__ ly,
                                                 i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                                                 i64* __restrict__ row_off, i64* __restrict__ lab_off,
-                                                i64* __restrict__ pad_off, i64* __restrict__ bnd_off,
-                                                int* __restrict__ seqmode, int* __restrict__ status,
-                                                float* __restrict__ costs) {
+                                                i64* __restrict__ pad_off, i64* __restrict__ slot_off,
+                                                i64* __restrict__ bnd_off, int* __restrict__ seqmode,
+                                                int* __restrict__ status, float* __restrict__ costs) {
     const int lane = threadIdx.x;
     i64 carry_r = 0, carry_l = 0, carry_p = 0, carry_b = 0;
     int flags = 0;
@@ -116,6 +116,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                     flags |= CWR_FLAG_U_TOO_LARGE;
                 }
                 pad_off[i] = ok ? ps : -1;
+                slot_off[i] = ps;
                 bnd_off[i] = bs;
                 seqmode[i] = 0;
             }
@@ -137,6 +138,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
         lab_off[N] = carry_l;
         if (pad_off) {
             pad_off[N] = carry_p;
+            slot_off[N] = carry_p;
             bnd_off[N] = carry_b;
         }
         if (R >= 0 && carry_r != R) flags |= CWR_FLAG_ROWS_MISMATCH;
@@ -148,10 +150,10 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
 }
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* bnd_off, int* seqmode, int* status,
-                   float* costs, hipStream_t stream) {
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode,
+                   int* status, float* costs, hipStream_t stream) {
     hipLaunchKernelGGL(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
-                       row_off, lab_off, pad_off, bnd_off, seqmode, status, costs);
+                       row_off, lab_off, pad_off, slot_off, bnd_off, seqmode, status, costs);
     return check_launch();
 }
 
@@ -615,6 +617,15 @@ struct LatticeView {
     i64 pad;
     int T, Up;
     bool linear, beta;
+    // value at `slot` of the strip that starts at slot `base`, written at step k of its walk
+    __device__ __forceinline__ double at_slot(i64 slot, i64 base, int k) const {
+        const double x = v[slot];
+        if (!linear) return x;
+        const int C = scale[(base >> 4) + (k / kPF)];
+        const int ex = __builtin_amdgcn_frexp_exp(x);
+        const float mant = (float)__builtin_amdgcn_frexp_mant(x);
+        return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
+    }
     __device__ __forceinline__ double log2_at(int t, int u) const {
         const i64 slot = pad + lattice_slot(t, u, T, Up);
         const double x = v[slot];
@@ -632,66 +643,110 @@ struct LatticeView {
     }
 };
 
+// One thread per lattice SLOT, so that a wave reads alpha, beta and the cell records of 64
+// neighbouring slots (consecutive addresses; a thread per compact row would touch one cache line
+// per lane, the strip layout being diagonal to the row order).  The two successors of cell (t,u)
+// sit one strip row further: same column (t+1,u) and next column (t,u+1); only the last column of a
+// strip looks into the next strip.  The 8-byte results are scattered to the row order.
 __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
                                                const i64* __restrict__ pad_off,
+                                               const i64* __restrict__ slot_off,
                                                const int* __restrict__ seqmode, int N, i64 R,
-                                               const int2* __restrict__ rowinfo, const LpCell* __restrict__ lp,
+                                               const LpCell* __restrict__ lp,
                                                const double* __restrict__ alpha, const double* __restrict__ beta,
                                                const int* __restrict__ scale_a, const int* __restrict__ scale_b,
                                                float2* __restrict__ grads, float* __restrict__ costs,
                                                int* __restrict__ status) {
-    const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
-    if (r >= R) return;
-    // the gather pass has already found the row's sequence
-    const int n = rowinfo[r].y;
-    RowInfo ri;
-    ri.n = -1;
-    if (n >= 0 && n < N) ri = place_row(r, n, R, row_off, lx, ly);
-    const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-    if (pad < 0) {
-        grads[r] = make_float2(0.f, 0.f);
-        return;
+    const i64 slot = (i64)blockIdx.x * 256 + threadIdx.x;
+    // the sequence whose slots hold this one: the last n with slot_off[n] <= slot (skipped
+    // sequences have no slots)
+    int n = 0;
+    if (N <= 64) {
+        // lane i holds slot_off[i]; a wave's 64 slots start in one sequence and cross few
+        // boundaries, so one ballot and a short loop replace a chain of dependent loads
+        const int lane = threadIdx.x & 63;
+        const i64 total = slot_off[N];
+        const i64 mine = lane < N ? slot_off[lane] : 0x7fffffffffffffffLL;
+        const i64 s0 = slot - lane;
+        n = __popcll(__ballot(mine <= s0)) - 1;
+        unsigned long long inside = __ballot(mine > s0 && mine <= s0 + 63);
+        while (inside) {
+            const int i = __ffsll((long long)inside) - 1;
+            inside &= inside - 1;
+            const i64 b = ((i64)__builtin_amdgcn_readlane((int)(mine >> 32), i) << 32) |
+                          (unsigned)__builtin_amdgcn_readlane((int)mine, i);
+            if (slot >= b) n = i;
+        }
+        if (slot >= total) return;
+    } else {
+        if (slot >= slot_off[N]) return;
+        int lo = 0, hi = N;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (slot_off[mid] <= slot) lo = mid; else hi = mid;
+        }
+        n = lo;
     }
-    const int T = ri.T, U = ri.U, t = ri.t, u = ri.u;
+    const i64 pad = pad_off[n];
+    if (pad < 0) return;
+    const int T = lx[n], U = ly[n];
     const int Up = U + 1;
     const int S = (Up + 63) >> 6;
-    const bool linear = seqmode[ri.n] == 0 && S <= kMaxWaves;
+    const i64 full = strip_rows(T, 64) * 64;
+    const i64 local = slot - pad;
+    i64 s64 = local / full;
+    const int s = (int)(s64 < S - 1 ? s64 : S - 1);
+    const int rem = (int)(local - (i64)s * full);
+    const int nl = s == S - 1 ? Up - (s << 6) : 64;
+    const int row = rem / nl;
+    const int l = rem - row * nl;
+    const int t = row - l - kRowShift, u = (s << 6) + l;
+    if (t < 0 || t >= T) return;  // padding
+    const i64 r = row_off[n] + (i64)t * Up + u;
+    if (r >= R) return;
+    const bool linear = seqmode[n] == 0 && S <= kMaxWaves;
     LatticeView A, Bv;
     A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear; A.beta = false;
     Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear; Bv.beta = true;
-    const double a = A.log2_at(t, u);
-    const LpCell cell = lp[pad + lattice_slot(t, u, T, Up)];
-    const float2 c = make_float2(cell.l_blank, cell.l_label);
+    const i64 base = pad + (i64)s * full;
+    const int q = t + l;
+    const double a = A.at_slot(slot, base, q);
+    const LpCell cell = lp[slot];
     const double b00 = Bv.log2_at(0, 0);
     // all values are base-2 logarithms
     float gb = 0.f, gl = 0.f;
     if (t < T - 1) {
-        gb = -fast_exp2((float)(a + Bv.log2_at(t + 1, u) + (double)c.x - b00));
+        gb = -fast_exp2((float)(a + Bv.at_slot(slot + nl, base, T + nl - 2 - (q + 1)) + (double)cell.l_blank - b00));
     } else if (u == U) {
-        gb = -fast_exp2((float)(a + (double)c.x - b00));
+        gb = -fast_exp2((float)(a + (double)cell.l_blank - b00));
     }
-    if (u < U) gl = -fast_exp2((float)(a + Bv.log2_at(t, u + 1) + (double)c.y - b00));
+    if (u < U) {
+        const double bn = l + 1 < nl ? Bv.at_slot(slot + nl + 1, base, T + nl - 2 - (q + 1)) : Bv.log2_at(t, u + 1);
+        gl = -fast_exp2((float)(a + bn + (double)cell.l_label - b00));
+    }
     grads[r] = make_float2(gb, gl);
     if (t == T - 1 && u == U) {
         // cwarp_cuda_rnnt_kernel.cu:353-366
-        double fa = a + (double)c.x;
+        double fa = a + (double)cell.l_blank;
         double fb = b00;
         double ratio = fabs(fa - fb) / fabs(fmax(fa, fb));
         if (ratio > 1e-3) {
             atomicOr(status, CWR_FLAG_FB_MISMATCH);
             fb = (fa + fb) * 0.5;
         }
-        costs[ri.n] = (float)(-fb * (double)kLn2);
+        costs[n] = (float)(-fb * (double)kLn2);
     }
 }
 
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs) {
     if (b.R == 0) return CWR_OK;
-    unsigned blocks = (unsigned)((b.R + 255) / 256);
-    hipLaunchKernelGGL(k_fill, dim3(blocks), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off, ws.pad_off,
-                       ws.seqmode, b.N, b.R, reinterpret_cast<const int2*>(rowinfo), ws.lp, ws.alpha, ws.beta,
-                       ws.scale_a, ws.scale_b, reinterpret_cast<float2*>(grads), costs, b.status);
+    const i64 slots = ws.slot_cap;  // the device knows the exact count; threads beyond it leave at once
+    if ((slots + 255) / 256 > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(k_fill, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
+                       ws.pad_off, ws.slot_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
+                       ws.scale_b, reinterpret_cast<float2*>(grads), costs, b.status);
+    (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
     return check_launch();
 }
 

@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
     LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ seqmode, int* __restrict__ status) {
+    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     // beyond 32 values per lane the register vector would be indexed through scratch memory:
     // the two entries are then read back from the row itself (it has just been fetched)
@@ -273,6 +273,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
         lse_out[r] = lse;
         rowinfo[r] = make_int2(lab, ri.n);
         if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
     }
 }
 
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
     LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ seqmode, int* __restrict__ status) {
+    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;   // rows per pass
     constexpr int ROWS = RP * NP;  // rows per wave
@@ -395,6 +396,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         lse_out[r] = res_lse;
         rowinfo[r] = make_int2(my_lab, ri.n);
         if (my_dst >= 0) lp[my_dst] = make_lp(res_b, res_l, res_lse, my_lab >= 0, seqmode + ri.n);
+        else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
     }
 }
 
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
     LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    int* __restrict__ seqmode, int* __restrict__ status) {
+    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     const int lane = threadIdx.x & 63;
     const i64 r = wave_first_row(1);
     if (r >= R) return;
@@ -429,6 +431,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
             lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        } else if (grads_skipped) {
+            grads_skipped[r] = make_float2(0.f, 0.f);
         }
         rowinfo[r] = make_int2(lab, ri.n);
     }
@@ -440,8 +444,8 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, int2* __restrict__ rowinfo, int* __restrict__ seqmode,
-    int* __restrict__ status) {
+    LpCell* __restrict__ lp, int2* __restrict__ rowinfo, float2* __restrict__ grads_skipped,
+    int* __restrict__ seqmode, int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;
     const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
@@ -454,6 +458,8 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
         const float xb = Elem<T>::to_f32(row[blank]);
         const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
         lp[dst] = make_lp(xb, xl, 0.f, lab >= 0, seqmode + ri.n);
+    } else if (grads_skipped) {
+        grads_skipped[r] = make_float2(0.f, 0.f);
     }
     rowinfo[r] = make_int2(lab, ri.n);
 }
@@ -640,21 +646,22 @@ constexpr bool kGradNT = true;
 static unsigned blocks_for_waves(i64 waves) { return (unsigned)((waves + kWavesPerBlock - 1) / kWavesPerBlock); }
 
 template <typename T>
-static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* rowinfo) {
+static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads) {
     const T* x = static_cast<const T*>(b.x);
     int2* ri = reinterpret_cast<int2*>(rowinfo);
+    float2* gz = reinterpret_cast<float2*>(grads);  // rows of skipped sequences get a zero record here
     if (b.R == 0) return CWR_OK;
     if (b.mode == CWR_MODE_LOGPROB) {
         unsigned blocks = (unsigned)((b.R + 255) / 256);
         hipLaunchKernelGGL((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
                            b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,
-                           ws.lp, ri, ws.seqmode, b.status);
+                           ws.lp, ri, gz, ws.seqmode, b.status);
         return check_launch();
     }
     int lpr = 0, k = 0;
     if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
 #define CWR_ARGS x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,   \
-                 b.blank, ws.lp, lse, ri, ws.seqmode, b.status
+                 b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status
         // grids are multiples of 8 workgroups, see logical_block
 #define CWR_ROW(KK)                                                                                  \
     if (lpr == 64 && k == KK) {                                                                      \
@@ -678,7 +685,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     }
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
-                       ws.pad_off, b.N, b.blank, ws.lp, lse, ri, ws.seqmode, b.status);
+                       ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);
     return check_launch();
 }
 
@@ -718,12 +725,12 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
     return check_launch();
 }
 
-int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo) {
+int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads) {
     switch (b.dtype) {
-        case CWR_F32: return gather_typed<float>(b, ws, lse, rowinfo);
-        case CWR_F16: return gather_typed<__half>(b, ws, lse, rowinfo);
-        case CWR_BF16: return gather_typed<bf16_t>(b, ws, lse, rowinfo);
-        case CWR_F64: return gather_typed<double>(b, ws, lse, rowinfo);
+        case CWR_F32: return gather_typed<float>(b, ws, lse, rowinfo, grads);
+        case CWR_F16: return gather_typed<__half>(b, ws, lse, rowinfo, grads);
+        case CWR_BF16: return gather_typed<bf16_t>(b, ws, lse, rowinfo, grads);
+        case CWR_F64: return gather_typed<double>(b, ws, lse, rowinfo, grads);
     }
     return CWR_ERR_DTYPE;
 }
