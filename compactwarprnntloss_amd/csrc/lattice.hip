@@ -9,14 +9,15 @@
 // Lattice walk: one wave owns a strip of 64 label positions of one sequence and walks it along
 // the anti-diagonals; at step q lane l holds cell (t = q - l, u = 64 s + l).  The neighbour in u
 // is the adjacent lane (one DPP wave shift), the neighbour in t is the lane's own previous value,
-// so a step needs no LDS and no barrier.  A lone wave issues one instruction every four cycles
+// so a step needs no barrier.  A lone wave issues one instruction every four to five cycles
 // whatever its kind, so the step is written for the smallest instruction count:
 //   - the strip layout (see lattice_slot) makes every step's access one row at a constant pitch:
 //     buffer instructions with a per-lane constant offset and a scalar row offset, no address
 //     arithmetic on the vector unit;
 //   - no lane is ever predicated: lanes that hold no cell read and write padding slots, and the
-//     recursion keeps them at the "no path" marker by itself (see sweep_strip);
-//   - values are base-2 logarithms, so log-sum-exp is v_exp_f32 / v_log_f32 without scaling.
+//     recursion keeps them at the "no path" marker by itself (see below);
+//   - the normal number system is the scaled linear domain (one fp64 add and two multiplies per
+//     cell); base-2 logarithms on the v_exp_f32 / v_log_f32 units are the fallback.
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
@@ -177,8 +178,8 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 //           checked that no log-prob of the sequence can push a value out of the fp64 range
 //           within one block (kLinMin, kLinMax).
 //   log     values are base-2 logarithms in fp64, (+) is max + log2(1 + 2^-|d|) on the fp32
-//           exp2/log2 units, (x) an add.  About 3.5x slower per step; used for the sequences the
-//           gather pass marked (extreme log-probs) and for those with more strips than waves.
+//           exp2/log2 units, (x) an add.  Used for the sequences the gather pass marked (extreme
+//           log-probs) and for those with more strips than waves.
 //
 // Lanes that hold no cell at a step are not masked:
 //   - before its first cell a lane holds "no path" (0, or -1e30 as a logarithm) in own and nbr';
