@@ -390,3 +390,15 @@ def test_full_size_configs_against_oracle(idx):
     np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
     np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
     assert float(np.abs(g.cpu().numpy() - ref["grad"]).max()) <= GRAD_ATOL
+
+
+@pytest.mark.parametrize("fused,V", [(True, 64), (True, 1024), (False, 40)])
+def test_more_than_64_sequences(fused, V):
+    """Batches beyond 64 sequences leave the in-register sequence tables (gather, fill) for the
+    search over the offset arrays."""
+    rng = np.random.default_rng(77)
+    N = 150
+    lx = rng.integers(1, 12, N)
+    ly = rng.integers(0, 9, N)
+    b = make_batch(lx, ly, V, seed=12, normalised=not fused)
+    check_case(b, fused, "1d")
