@@ -17,9 +17,10 @@ constexpr float kLn2 = 0.6931471805599453f;
 // "no path" marker of the lattice recursions.  Finite, so that marker - marker = 0 instead of NaN.
 constexpr double kNeg = -1.0e30;
 constexpr float kLpFloor = -1.0e30f;  // gathered log-probs are clamped to this (keeps -inf logits finite)
-// The scaled linear-domain walk renormalises every kPF = 16 steps to a maximum of 2^kLinTarget.
-// Inside a block a value can shrink by 2^(16*kLinMin) and grow by 2^(16*(kLinMax+1)), which must
-// stay inside the fp64 range: 800 - 16*100 = -800 > -1022 and 800 + 16*9 = 944 < 1023.
+// The scaled linear-domain walk renormalises every kPF = 16 steps to a maximum of 2^kLinTarget
+// per column.  Inside a block a value can shrink by 2^(16*kLinMin) and grow by
+// 2^(16*(kLinMax+1)), which stays inside the fp64 range: 800 - 16*100 = -800 > -1022 and
+// 800 + 16*9 = 944 < 1023.
 constexpr float kLinMin = -100.0f;  // base-2 log-probs below this ...
 constexpr float kLinMax = 8.0f;     // ... or above this send the sequence to the log-domain walk
 constexpr int kLinTarget = 800;
@@ -29,7 +30,8 @@ constexpr int kLinTarget = 800;
 // ---------------------------------------------------------------------------------------------
 constexpr int DPP_QUAD_XOR1 = 0xB1;    // quad_perm:[1,0,3,2]
 constexpr int DPP_QUAD_XOR2 = 0x4E;    // quad_perm:[2,3,0,1]
-constexpr int DPP_ROW_SHR = 0x110;     // + n
+constexpr int DPP_ROW_SHL = 0x100;     // + n: lane i reads lane i+n of its row of 16
+constexpr int DPP_ROW_SHR = 0x110;     // + n: lane i reads lane i-n of its row of 16
 constexpr int DPP_WAVE_SHL1 = 0x130;   // lane i reads lane i+1
 constexpr int DPP_WAVE_SHR1 = 0x138;   // lane i reads lane i-1
 constexpr int DPP_ROW_MIRROR = 0x140;

@@ -38,11 +38,12 @@ struct Workspace {
     i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
     i64* slot_off;  // N+1  the same running sum without the -1 marks (monotone: searchable)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
-    int* seqmode;   // N+1  per sequence: 0 = walk in the scaled linear domain, 1 = in the log domain
+    int* seqmode;   // N+1  per sequence: 0 = walked in the scaled linear domain; bit 0 = in the log domain
+                    //      (gather's verdict), bits 1 / 2 = alpha / beta repeated in the log domain
     LpCell* lp;     // slot_cap  gathered (blank, label) log-probabilities and probabilities
-    double* alpha;  // slot_cap  log2(alpha), or alpha * 2^scale_a[block] (see seqmode)
+    double* alpha;  // slot_cap  log2(alpha), or alpha * 2^scale_a[block][column] (see seqmode)
     double* beta;   // slot_cap
-    int* scale_a;   // slot_cap/16+1  exponent of each 16-step block of a strip's alpha walk
+    int* scale_a;   // slot_cap/16+1  per strip: exponent of each (16-step block, column) of the alpha walk
     int* scale_b;   // same for beta
     double* bnd_a;  // bnd_cap   alpha values handed from one 64-label strip to the next
     double* bnd_b;  // bnd_cap   same for beta

@@ -255,9 +255,65 @@ __device__ __forceinline__ double exp2_f64(float x) { return (double)fast_exp2(x
 // the dependent chain.  The values that enter from the previous strip are prepared once per block
 // by lanes 0..kPF-1 (lane j: the value entering at step k0+j) and picked per step with a readlane.
 
+// Zeroes the triangle of padding records a direction reads before a lane's first cell.  A zero
+// record is "probability 0" for the linear walk and "log-prob 0" for the log walk; both keep a
+// lane that holds "no path" there (junk in those records could be a NaN, which nothing survives).
+template <bool BETA>
+__device__ __forceinline__ void clear_leading(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
+    const int p16 = nl * 16;
+#pragma unroll 4
+    for (int j = 0; j < nl - 1; ++j) {
+        const int row = (BETA ? T + j : j) + kRowShift;
+        const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
+        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
+    }
+    __threadfence_block();
+}
+
+// The linear walk wants every record it reads outside a lane's cells to be zero, before AND after
+// them (and for the up to kPF-1 steps it runs past its last diagonal): then a lane outside its
+// cells holds exactly 0, never junk, and "non-zero" means "a cell" for the range check below.
+// Both directions of a sequence clear the same records; nothing else is ever written to them.
+template <bool BETA>
+__device__ __forceinline__ void clear_around(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
+    const int p16 = nl * 16;
+    const int Q = T + nl - 1;
+    const int vo = lane < nl ? lane * 16 : kOob;
+    // row j of the cells' bounding box: lanes > j have not started; in row T+j lanes <= j have
+    // finished; one store covers both (the per-lane offset picks the row)
+#pragma unroll 4
+    for (int j = 0; j < nl - 1; ++j)
+        buf_store_zero16(r_cell, lane < nl ? lane * 16 + (lane > j ? 0 : T * p16) : kOob, (j + kRowShift) * p16);
+#pragma unroll 4
+    for (int j = 1; j <= kPF; ++j)
+        buf_store_zero16(r_cell, vo, (BETA ? kRowShift - j : Q - 1 + j + kRowShift) * p16);
+    __threadfence_block();
+}
+
+// Range check of the linear walk.  Every kCheckEvery-th step all cell values must lie inside
+// [2^kLowExp, 2^kHighExp) at their lane's scale; otherwise the walk reports the direction as
+// unsafe and it is walked again in the log domain.  In between, a value descends from checked ones
+// through at most kCheckEvery products with factors in [2^kLinMin, 2^(kLinMax+1)], so inside the
+// bounds no product can leave the normal fp64 range (-600 - 4*100 > -1022, 980 + 4*9 < 1023): the
+// results are then exact up to rounding, whatever the spread of magnitudes across the lattice.
+constexpr int kCheckEvery = 4;
+constexpr int kLowExp = -600;
+constexpr int kHighExp = 980;
+constexpr unsigned kLowHigh = (unsigned)(1023 + kLowExp) << 20;    // high word of 2^kLowExp
+constexpr unsigned kHighHigh = (unsigned)(1023 + kHighExp) << 20;  // high word of 2^kHighExp
+
 // ---- scaled linear-domain walk (strips concurrent, LDS rings) -------------------------------
+// Every LANE carries its own scale: the values of column u are probabilities times 2^C[u], with
+// C[u] renewed at the start of every block of kPF steps so that the larger of the lane's own value
+// and of what its neighbour is about to hand over sits at 2^kLinTarget.  A value arriving from the
+// neighbouring lane is brought to the lane's scale by one v_ldexp_f64 with the (block-constant)
+// difference of the two scales.  Like a logarithm, this loses nothing across columns, however far
+// apart their magnitudes are: the only thing that can underflow is a summand that is negligible
+// next to the other summand of the SAME cell.  Within a block a lane's value can still drift out
+// of the fp64 range (a run of extreme factors, or a much larger magnitude arriving from several
+// columns away), which the range check catches.  Returns false when the check failed.
 template <bool BETA, bool HAS_IN, bool HAS_OUT>
-__device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const bool seed, const int in_shift,
+__device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const bool seed, const int in_shift,
                                                 const int out_shift, const LpCell* lp_strip,
                                                 double* out_strip, int* scale_strip, const Ring rin,
                                                 const Ring rout, int* status) {
@@ -265,25 +321,19 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    const int p16 = nl * 16, p8 = nl * 8;
+    const int p16 = nl * 16, p8 = nl * 8, p4 = nl * 4;
     const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
-    const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * 4);
+    const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * p4);
     const int vo_p = lane < nl ? lane * 16 : kOob;  // the two probabilities of a record
     const int vo = lane < nl ? lane * 8 : kOob;
-    const int vo_sc = lane == 0 ? 0 : kOob;
+    const int vo_sc = lane < nl ? lane * 4 : kOob;
     constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 64 wide
     constexpr int out_lane = BETA ? 0 : 63;
     double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
 
-    // clear the triangle of padding records this direction reads before a lane's first cell
-    for (int j = 0; j < nl - 1; ++j) {
-        const int row = (BETA ? T + j : j) + kRowShift;
-        const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
-        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
-    }
-    __threadfence_block();
+    clear_around<BETA>(r_cell, T, nl, lane);
 
     const int row0 = (BETA ? Q - 1 : 0) + kRowShift;  // row of step 0
     int qi = row0;                                    // row of the current step
@@ -291,7 +341,8 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
     float2 ring[kPF];                                 // (blank, label) probabilities, rows mi .. mi+dq*(kPF-1)
 #pragma unroll
     for (int j = 0; j < kPF; ++j) ring[j] = buf_load_f2(r_cell, vo_p, (mi + dq * j) * p16);
-    int C = kLinTarget;
+    int C = kLinTarget;  // this lane's scale exponent
+    int d = 0;           // C minus the scale exponent of the lane the neighbour values come from
     // alpha[0][0] = 1; beta[T-1][U] = blank probability of that cell
     double own = 0.0;
     if (BETA) {
@@ -307,6 +358,7 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
     double mul_own = (double)ring[0].x;
     double mul_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, ring[0].y) : ring[0].y);
     const double in_mask = lane == in_lane ? 1.0 : 0.0;
+    unsigned lo_seen = 0xffffffffu, hi_seen = 0u;  // extremes of the cell values' high words (zero excluded)
     // beta hands on plain beta(t,u+1); the receiving edge column applies its own L(t,u), fetched
     // one block ahead by the lanes that prepare the incoming entries
     const int jl = lane & (kPF - 1);
@@ -318,11 +370,12 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
         if (HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
         if (HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
         keep_order();
-        // Renormalise.  Only lanes that still have cells count: a lane past its last cell (and a
-        // lane beyond the strip's width) carries junk of any magnitude.
-        const int first_step = BETA ? nl - 1 - lane : lane;
-        const bool alive = lane < nl && k0 - first_step < T;
-        int m = alive ? max(exponent_of(own), exponent_of(pass)) : kNoExp;
+        // Renew the scales.  True magnitude (binary exponent minus scale) of what the lane holds,
+        // of what it will hand over and of what its neighbour will hand over next:
+        const int t_own = own != 0.0 ? __builtin_amdgcn_frexp_exp(own) - C : kNoExp;
+        const int t_pass = pass != 0.0 ? __builtin_amdgcn_frexp_exp(pass) - C : kNoExp;
+        int t = max(max(t_own, t_pass),
+                    BETA ? dpp_i32<DPP_WAVE_SHL1>(kNoExp, t_pass) : dpp_i32<DPP_WAVE_SHR1>(kNoExp, t_pass));
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
@@ -336,27 +389,63 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
             const bool ok = k0 + jl < T && ev != 0.0;
             cp = (int)en.y;
             e_lane = ok ? ev : 0.0;
-            if (ok) m = max(m, __builtin_amdgcn_frexp_exp(ev) + C - cp);
+            // the largest of the kPF entries (they sit in every row of 16 lanes), for the edge lane
+            int te = ok ? __builtin_amdgcn_frexp_exp(ev) - cp : kNoExp;
+            te = max(te, dpp_i32<DPP_QUAD_XOR1>(kNoExp, te));
+            te = max(te, dpp_i32<DPP_QUAD_XOR2>(kNoExp, te));
+            te = max(te, dpp_i32<DPP_ROW_HALF_MIRROR>(kNoExp, te));
+            te = max(te, dpp_i32<DPP_ROW_MIRROR>(kNoExp, te));
+            if (lane == in_lane) t = max(t, te);
         }
-        const int M = wave_max_i32(m);
-        if (M > kNoExp / 2) {
-            const int delta = kLinTarget - M;
-            own = __builtin_ldexp(own, delta);
-            pass = __builtin_ldexp(pass, delta);
-            C += delta;
+        // Whatever reaches a lane during this block was, at its start, in one of the kPF lanes the
+        // values come from (or enters through the edge lane, counted above): take the largest
+        // magnitude over that window, so that nothing arriving can exceed 2^(kLinTarget + kPF*
+        // (kLinMax+1)).  Window used: the lanes before it in its row of 16 and the whole row before.
+        if (BETA) {
+            t = max(t, dpp_i32<DPP_ROW_SHL + 1>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 2>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 4>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 8>(kNoExp, t));
+            const int next_row = __shfl(t, (lane | 15) + 1 > 63 ? lane : (lane | 15) + 1);
+            if (lane < 48) t = max(t, next_row);
+        } else {
+            t = max(t, dpp_i32<DPP_ROW_SHR + 1>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 2>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 4>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 8>(kNoExp, t));
+            const int prev_row = __shfl(t, lane < 16 ? lane : (lane & ~15) - 1);
+            if (lane >= 16) t = max(t, prev_row);
         }
-        if (HAS_IN) e_lane = __builtin_ldexp(e_lane, C - cp);
-        buf_store_i32(r_sc, vo_sc, blk * 4, C);
-        const double Cd = (double)C;
+        const bool empty = t <= kNoExp / 2;
+        int Cn = empty ? C : kLinTarget - t;
+        // a lane that holds nothing yet takes the scale of the lane that started last: whatever
+        // reaches it during this block has come from there, through at most kPF products
+        const int started = BETA ? nl - k0 : k0 - 1;
+        const int last = started < 0 ? 0 : (started > nl - 1 ? nl - 1 : started);
+        const int Cref = __builtin_amdgcn_readlane(Cn, last);
+        Cn = empty ? Cref : Cn;
+        own = __builtin_ldexp(own, Cn - C);
+        pass = __builtin_ldexp(pass, Cn - C);
+        C = Cn;
+        d = C - (BETA ? dpp_i32<DPP_WAVE_SHL1>(C, C) : dpp_i32<DPP_WAVE_SHR1>(C, C));
+        if (lane >= nl) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
+        if (HAS_IN) e_lane = __builtin_ldexp(e_lane, __builtin_amdgcn_readlane(C, in_lane) - cp);
+        buf_store_i32(r_sc, vo_sc, blk * p4, C);
+        const double Cd = (double)__builtin_amdgcn_readlane(C, out_lane);
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
             const float2 cn = buf_load_f2(r_cell, vo_p, (mi + dq * kPF) * p16);
             double o = own;
             if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own);
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(nbr, pass) : dpp_f64<DPP_WAVE_SHR1>(nbr, pass);
-            const double a = o + nbr;
+            const double a = o + __builtin_ldexp(nbr, d);
             own = a * mul_own;
             pass = a * mul_pass;
+            if (j % kCheckEvery == 0) {
+                const unsigned h = (unsigned)__double2hiint(a);
+                lo_seen = min(lo_seen, h - 1u);  // zero wraps to the top and drops out
+                hi_seen = max(hi_seen, h);
+            }
             buf_store_d(r_out, vo, qi * p8, a);
             if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = make_double2(BETA ? a : pass, Cd);
             const float2 nx = ring[(j + 1) % kPF];
@@ -374,6 +463,7 @@ __device__ __forceinline__ void sweep_strip_lin(const int T, const int nl, const
         if (HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    return __ballot(lo_seen < kLowHigh - 1u || hi_seen >= kHighHigh) == 0;
 }
 
 // ---- log-domain walk ------------------------------------------------------------------------
@@ -401,12 +491,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
 
-    for (int j = 0; j < nl - 1; ++j) {
-        const int row = (BETA ? T + j : j) + kRowShift;
-        const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
-        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
-    }
-    __threadfence_block();
+    clear_leading<BETA>(r_cell, T, nl, lane);
 
     const int row0 = (BETA ? Q - 1 : 0) + kRowShift;
     int qi = row0;
@@ -488,13 +573,13 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
 }
 
 template <bool BETA>
-__device__ __forceinline__ void lin_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
+__device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
                                              int out_shift, const LpCell* lp, double* out, int* sc, Ring rin,
                                              Ring rout, int* status) {
-    if (has_in && has_out) sweep_strip_lin<BETA, true, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    else if (has_in) sweep_strip_lin<BETA, true, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    else if (has_out) sweep_strip_lin<BETA, false, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    else sweep_strip_lin<BETA, false, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_in && has_out) return sweep_strip_lin<BETA, true, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_in) return sweep_strip_lin<BETA, true, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_out) return sweep_strip_lin<BETA, false, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    return sweep_strip_lin<BETA, false, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
 }
 
 template <bool BETA, bool CONC>
@@ -518,11 +603,12 @@ constexpr int kMaxWaves = 8;
 
 __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
-    const i64* __restrict__ bnd_off, const int* __restrict__ seqmode, const LpCell* lp, double* alpha,
+    const i64* __restrict__ bnd_off, int* seqmode, const LpCell* lp, double* alpha,
     double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int* status) {
     __shared__ double2 s_ring[kMaxWaves - 1][2 * kRing + 64];
     __shared__ int s_produced[kMaxWaves];
     __shared__ int s_consumed[kMaxWaves];
+    __shared__ volatile int s_unsafe;
     const int n = blockIdx.x;
     const int dir = beta_only ? 1 : (int)blockIdx.y;
     const int W = blockDim.x >> 6;
@@ -532,6 +618,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         s_produced[threadIdx.x] = 0;
         s_consumed[threadIdx.x] = 0;
     }
+    if (threadIdx.x == 0) s_unsafe = 0;
     __syncthreads();
     const i64 pad = pad_off[n];
     if (pad < 0) return;
@@ -545,10 +632,12 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     Ring none;
     none.slots = nullptr; none.produced = nullptr; none.consumed = nullptr;
 
-    if (S <= W) {
+    const bool concurrent = S <= W;
+    const bool linear = concurrent && (seqmode[n] & 1) == 0;  // the gather pass's verdict on the log-probs
+    if (concurrent) {
         // position p in the order of the walk: alpha strip p, beta strip S-1-p
-        if (w >= S) return;
-        const int p = w;
+        const bool active = w < S;
+        const int p = active ? w : 0;
         const int s = dir ? S - 1 - p : p;
         const int nl = s == S - 1 ? nl_last : 64;
         const i64 base = pad + (i64)s * full_strip;
@@ -561,16 +650,24 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
         const int out_shift = dir ? nl - 1 : 63;
         const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
-        const bool linear = seqmode[n] == 0;
-        if (linear) {
-            int* sc = scale + (base >> 4);
-            if (dir == 0) lin_dispatch<false>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
-            else lin_dispatch<true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
-        } else {
+        if (!linear) {
+            if (!active) return;
             if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
             else log_dispatch<true, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+            return;
         }
-        return;
+        bool safe = true;
+        if (active) {
+            int* sc = scale + (base >> 4);
+            safe = dir == 0 ? lin_dispatch<false>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status)
+                            : lin_dispatch<true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
+        }
+        if (!safe && lane == 0) s_unsafe = 1;
+        __syncthreads();
+        if (s_unsafe == 0 || w != 0) return;
+        // Some strip of this direction left the range the linear walk is exact in: wave 0 walks
+        // the whole direction again, strip by strip, in the log domain (below).
+        if (lane == 0) atomicOr(&seqmode[n], dir ? 4 : 2);
     }
 
     if (w != 0) return;
@@ -610,6 +707,12 @@ int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
 // ---------------------------------------------------------------------------------------------
 // per-row gradient w.r.t. the gathered log-probs, and the costs
 // ---------------------------------------------------------------------------------------------
+// Walk-mode word of a sequence: bit 0 = the gather pass found log-probs the linear walk cannot
+// carry; bit 1 / bit 2 = the alpha / beta walk left the range it is exact in and was done again in
+// the log domain.  More strips than a workgroup has waves always means the log domain.
+__device__ __forceinline__ bool linear_alpha(int mode, int S) { return (mode & 3) == 0 && S <= kMaxWaves; }
+__device__ __forceinline__ bool linear_beta(int mode, int S) { return (mode & 5) == 0 && S <= kMaxWaves; }
+
 // Base-2 logarithm of the lattice value stored for cell (t,u): either stored as such (log walk),
 // or as value * 2^C with C recorded per block of kPF steps of the strip's walk (linear walk).
 struct LatticeView {
@@ -618,11 +721,12 @@ struct LatticeView {
     i64 pad;
     int T, Up;
     bool linear, beta;
-    // value at `slot` of the strip that starts at slot `base`, written at step k of its walk
-    __device__ __forceinline__ double at_slot(i64 slot, i64 base, int k) const {
+    // value at `slot`, column l of the nl-wide strip that starts at slot `base`, written at step k
+    // of its walk
+    __device__ __forceinline__ double at_slot(i64 slot, i64 base, int k, int nl, int l) const {
         const double x = v[slot];
         if (!linear) return x;
-        const int C = scale[(base >> 4) + (k / kPF)];
+        const int C = scale[(base >> 4) + (k / kPF) * nl + l];
         const int ex = __builtin_amdgcn_frexp_exp(x);
         const float mant = (float)__builtin_amdgcn_frexp_mant(x);
         return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
@@ -636,7 +740,7 @@ struct LatticeView {
         const int q = t + l;
         const int k = beta ? (T + nl - 2 - q) : q;
         const i64 base = pad + (i64)s * strip_rows(T, 64) * 64;
-        const int C = scale[(base >> 4) + (k / kPF)];
+        const int C = scale[(base >> 4) + (k / kPF) * nl + l];
         // log2 x = exponent + log2(mantissa), mantissa in [0.5, 1)
         const int ex = __builtin_amdgcn_frexp_exp(x);
         const float mant = (float)__builtin_amdgcn_frexp_mant(x);
@@ -706,24 +810,24 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
     if (t < 0 || t >= T) return;  // padding
     const i64 r = row_off[n] + (i64)t * Up + u;
     if (r >= R) return;
-    const bool linear = seqmode[n] == 0 && S <= kMaxWaves;
+    const int mode = seqmode[n];
     LatticeView A, Bv;
-    A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear; A.beta = false;
-    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear; Bv.beta = true;
+    A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
+    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
     const i64 base = pad + (i64)s * full;
     const int q = t + l;
-    const double a = A.at_slot(slot, base, q);
+    const double a = A.at_slot(slot, base, q, nl, l);
     const LpCell cell = lp[slot];
     const double b00 = Bv.log2_at(0, 0);
     // all values are base-2 logarithms
     float gb = 0.f, gl = 0.f;
     if (t < T - 1) {
-        gb = -fast_exp2((float)(a + Bv.at_slot(slot + nl, base, T + nl - 2 - (q + 1)) + (double)cell.l_blank - b00));
+        gb = -fast_exp2((float)(a + Bv.at_slot(slot + nl, base, T + nl - 2 - (q + 1), nl, l) + (double)cell.l_blank - b00));
     } else if (u == U) {
         gb = -fast_exp2((float)(a + (double)cell.l_blank - b00));
     }
     if (u < U) {
-        const double bn = l + 1 < nl ? Bv.at_slot(slot + nl + 1, base, T + nl - 2 - (q + 1)) : Bv.log2_at(t, u + 1);
+        const double bn = l + 1 < nl ? Bv.at_slot(slot + nl + 1, base, T + nl - 2 - (q + 1), nl, l + 1) : Bv.log2_at(t, u + 1);
         gl = -fast_exp2((float)(a + bn + (double)cell.l_label - b00));
     }
     grads[r] = make_float2(gb, gl);
@@ -763,7 +867,7 @@ __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ l
     if (pad < 0) return;  // NaN already set by k_offsets
     LatticeView Bv;
     Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
-    Bv.linear = seqmode[n] == 0 && ((Bv.Up + 63) >> 6) <= kMaxWaves;
+    Bv.linear = linear_beta(seqmode[n], (Bv.Up + 63) >> 6);
     costs[n] = (float)(-Bv.log2_at(0, 0) * (double)kLn2);
 }
 
@@ -797,9 +901,9 @@ __global__ __launch_bounds__(256) void k_export(const int* __restrict__ lx, cons
     double a = 0.0, b = 0.0;
     if (pad >= 0 && t < T && u < Up) {
         LatticeView A, Bv;
-        const bool linear = seqmode[n] == 0 && ((Up + 63) >> 6) <= kMaxWaves;
-        A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear; A.beta = false;
-        Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear; Bv.beta = true;
+        const int mode = seqmode[n], S = (Up + 63) >> 6;
+        A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
+        Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
         if (alphas_out) a = A.log2_at(t, u) * 0.6931471805599453;
         b = Bv.log2_at(t, u) * 0.6931471805599453;
     }

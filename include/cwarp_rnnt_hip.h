@@ -87,13 +87,16 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
  *      log2 P(label)
  *   1  alpha, 2  beta: one fp64 per cell
  *   3  pad_off: N+1 int64, first cell slot of each sequence, -1 for a skipped sequence
- *   4  seqmode: N+1 int32 (N used); 0 = the sequence was walked in the scaled linear domain,
- *      non-zero = in the log domain (also used when it has more than 8 strips of 64 labels)
+ *   4  seqmode: N+1 int32 (N used), how the sequence was walked.  0 = both directions in the
+ *      scaled linear domain; bit 0 = both in the log domain (log-probs outside what the linear
+ *      walk carries); bit 1 / bit 2 = alpha / beta was walked again in the log domain.  A sequence
+ *      with more than 8 strips of 64 labels is always in the log domain.
  *   5  scale_a, 6  scale_b: int32 scale exponents of the linear-domain walk
  * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U).
- * Log-domain sequences hold base-2 logarithms (multiply by ln 2).  Linear-domain sequences hold
- * value * 2^C: for strip s = u/64 of width nl = min(64, U+1-64s), lane l = u%64, the walk step is
- * k = t+l (alpha) or T+nl-2-(t+l) (beta) and C = scale[(pad_off[n] + s*(T+127)*64)/16 + k/16]. */
+ * Log-domain values are base-2 logarithms (multiply by ln 2).  Linear-domain values are
+ * value * 2^C: for strip s = u/64 of width nl = min(64, U+1-64s), column l = u%64, the walk step is
+ * k = t+l (alpha) or T+nl-2-(t+l) (beta) and
+ * C = scale[(pad_off[n] + s*(T+127)*64)/16 + (k/16)*nl + l].  cwr_export_lattice does this. */
 int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes);
 int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
 

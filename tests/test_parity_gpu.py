@@ -402,3 +402,86 @@ def test_more_than_64_sequences(fused, V):
     ly = rng.integers(0, 9, N)
     b = make_batch(lx, ly, V, seed=12, normalised=not fused)
     check_case(b, fused, "1d")
+
+
+# ----------------------------------------------------------------------------- number systems of the lattice walk
+def _walk_modes(st):
+    """Per-sequence walk-mode words of a forward call (workspace section 4)."""
+    import ctypes as C
+    lib = _pkg()._lib.load()
+    off, nbytes = C.c_size_t(), C.c_size_t()
+    assert lib.cwr_workspace_section(st.N, st.R, st.max_u, 4, C.byref(off), C.byref(nbytes)) == 0
+    return st.workspace[off.value: off.value + 4 * st.N].view(torch.int32).cpu().numpy()
+
+
+def _logprob_case(lx, ly, V, blank_nats, label_nats=None, seed=1):
+    b = make_batch(lx, ly, V, seed=seed, normalised=True)
+    x = b["x"].clone()
+    x[:, 0] = blank_nats
+    if label_nats is not None:
+        x[:, 1:] = label_nats
+    b["x"] = x
+    b["x_ref"] = x.double().numpy()
+    return b
+
+
+@pytest.mark.parametrize("blank_nats", [-10.0, -30.0, -45.0, -62.0])
+def test_columns_of_very_different_magnitude_stay_exact(blank_nats):
+    """A blank that is improbable everywhere makes neighbouring label positions differ by that
+    factor, so a diagonal of 60 cells spans thousands of bits.  The linear-domain walk carries
+    one scale per column and must still be exact (a single scale per wave is not)."""
+    b = _logprob_case([40, 120], [60, 50], 8, blank_nats)
+    pkg = _pkg()
+    dev = torch.device("cuda:0")
+    xs = b["x"].to(dev)
+    lx, ly = torch.from_numpy(b["lx"]).to(dev), torch.from_numpy(b["ly"]).to(dev)
+    ys = torch.from_numpy(b["yp"]).to(dev)
+    costs, st = pkg.rnnt_forward(xs, lx, ys, ly, 0, False)
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "logprob")
+    assert int(st.status[0].item()) == 0
+    np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
+    assert not _walk_modes(st).any()        # all of it in the linear domain
+
+
+def test_walk_leaves_the_linear_domain_when_its_range_check_fails():
+    """Labels of probability 2^-95 next to blanks of probability ~1 put every label position 95
+    bits below the one that feeds it; a column then sits more than 600 bits below the largest
+    magnitude that can reach it within a block of steps, the range check of the linear walk fails,
+    and the direction is walked again in the log domain.  The result must not care."""
+    lx, ly = [70, 30], [20, 90]
+    b = _logprob_case(lx, ly, 6, -0.1, -66.0)
+    pkg = _pkg()
+    dev = torch.device("cuda:0")
+    xs = b["x"].to(dev)
+    lxd, lyd = torch.from_numpy(b["lx"]).to(dev), torch.from_numpy(b["ly"]).to(dev)
+    ys = torch.from_numpy(b["yp"]).to(dev)
+    costs, st = pkg.rnnt_forward(xs, lxd, ys, lyd, 0, False)
+    modes = _walk_modes(st)
+    assert (modes & 1 == 0).all() and (modes & 6 == 6).all()      # both directions were done again
+    assert int(st.status[0].item()) == 0
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "logprob")
+    np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
+    # the alpha / beta export reads the log-domain values of such a sequence
+    alphas, betas = pkg.lattice_state(st, lxd, lyd, max(lx), max(ly) + 1)
+    off = orc.row_offsets_i64(b["lx"], b["ly"])
+    g = orc.gather(b["x_ref"], b["lx"], b["yp"], b["ly"], 0)
+    for n, (T, U) in enumerate(zip(lx, ly)):
+        lp = g[off[n]:off[n + 1]].reshape(T, U + 1, 2)
+        np.testing.assert_allclose(alphas[n, :T, :U + 1].cpu().numpy(), orc.alphas(lp), rtol=1e-6, atol=1e-3)
+        np.testing.assert_allclose(betas[n, :T, :U + 1].cpu().numpy(), orc.betas(lp), rtol=1e-6, atol=1e-3)
+
+
+def test_uniform_lattice_of_tiny_probabilities_matches_the_closed_form():
+    """One log-probability c = -66 nats (2^-95) everywhere: the loss is (T+U)*(-c) minus the log
+    of the number of paths, C(T+U-1, U); sixteen steps shrink a value by 2^-1523, which the linear
+    walk's per-block rescaling must carry."""
+    c = -66.0
+    lx, ly = [70, 30], [20, 90]
+    b = _logprob_case(lx, ly, 6, c, c)
+    dev = run_device(b, False)
+    want = [-(T + U) * c - (math.lgamma(T + U) - math.lgamma(U + 1) - math.lgamma(T)) for T, U in zip(lx, ly)]
+    np.testing.assert_allclose(dev["costs"], want, rtol=LOSS_RTOL)
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "logprob")
+    np.testing.assert_allclose(dev["G"], ref["G"], rtol=0, atol=GRAD_ATOL)
