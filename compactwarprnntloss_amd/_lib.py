@@ -39,6 +39,10 @@ SIGNATURES = {
                               _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
     "cwr_loss": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                            _p, _sz, _p, _p, _p, _p, _p]),
+    "cwr_forward_reduced": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
+                                      _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "cwr_loss_reduced": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
+                                   _p, _sz, _p, _p, _p, _p, _p, _p]),
     "cwr_backward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int,
                                _p, _p, _p, _p, _p, _p, _i64, C.c_float, _p, _p]),
     "cwr_rowinfo": (C.c_int, [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _p, _p, _p, _p]),

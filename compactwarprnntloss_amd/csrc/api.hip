@@ -133,7 +133,7 @@ using namespace cwr;
 
 extern "C" {
 
-int cwr_version(void) { return 110; }
+int cwr_version(void) { return 120; }
 
 const char* cwr_strerror(int status) {
     switch (status) {
@@ -173,7 +173,7 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
         misaligned(status, 4))
         return CWR_ERR_ALIGN;
     return launch_offsets(lx, ly, N, R, 0, 0, 0, reinterpret_cast<i64*>(row_off),
-                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, nullptr, nullptr, status, nullptr,
+                          reinterpret_cast<i64*>(lab_off), nullptr, nullptr, nullptr, nullptr, status, nullptr, nullptr,
                           static_cast<hipStream_t>(stream));
 }
 
@@ -181,7 +181,7 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
                         int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse, float* grads,
-                        float* costs, void* stream, bool with_grad) {
+                        float* costs, float* reduced, void* stream, bool with_grad) {
     int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
     if (rc != CWR_OK) return rc;
     if (max_u < 0) return CWR_ERR_SHAPE;
@@ -192,14 +192,15 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (R > 0 && (!rowinfo || (with_grad && !grads))) return CWR_ERR_NULL;
     if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
         misaligned(rowinfo, 8) ||
-        misaligned(grads, 8) || misaligned(costs, 4) || misaligned(workspace, 256))
+        misaligned(grads, 8) || misaligned(costs, 4) || misaligned(reduced, 4) || misaligned(workspace, 256))
         return CWR_ERR_ALIGN;
     Workspace ws;
     if (!carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws)) return CWR_ERR_SHAPE;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
-                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.slot_off, ws.bnd_off, ws.seqmode, status, costs, s);
+                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.slot_off, ws.bnd_off, ws.seqmode, status, costs,
+                        reduced, s);
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
@@ -207,8 +208,8 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (rc != CWR_OK) return rc;
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;
-    if (with_grad) return launch_fill(b, ws, rowinfo, grads, costs);
-    return launch_cost_from_beta(b, ws, costs);
+    if (with_grad) return launch_fill(b, ws, rowinfo, grads, costs, reduced);
+    return launch_cost_from_beta(b, ws, costs, reduced);
 }
 
 int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
@@ -216,13 +217,25 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* l
                 int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
                 int32_t* status, int32_t* rowinfo, float* lse, float* grads, float* costs, void* stream) {
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
-                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, stream, true);
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream,
+                        true);
 }
 
-int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
-             const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
-             int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
-             int32_t* status, float* costs, void* stream) {
+int cwr_forward_reduced(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                        const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                        int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
+                        int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse, float* grads,
+                        float* costs, float* reduced, void* stream) {
+    if (!reduced) return CWR_ERR_NULL;
+    return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, reduced, stream,
+                        true);
+}
+
+static int loss_impl(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                     const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                     int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
+                     int32_t* status, float* costs, float* reduced, void* stream) {
     // the gather still needs somewhere to put lse and the row records: the workspace's aux section
     Workspace ws;
     float* lse = nullptr;
@@ -233,8 +246,25 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, 
         lse = reinterpret_cast<float*>(ws.aux + (size_t)R * 8);
     }
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
-                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, nullptr, costs, stream,
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, nullptr, costs, reduced, stream,
                         false);
+}
+
+int cwr_loss(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+             const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+             int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
+             int32_t* status, float* costs, void* stream) {
+    return loss_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                     workspace_bytes_, row_off, lab_off, status, costs, nullptr, stream);
+}
+
+int cwr_loss_reduced(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                     const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                     int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off, int64_t* lab_off,
+                     int32_t* status, float* costs, float* reduced, void* stream) {
+    if (!reduced) return CWR_ERR_NULL;
+    return loss_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                     workspace_bytes_, row_off, lab_off, status, costs, reduced, stream);
 }
 
 int cwr_backward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,

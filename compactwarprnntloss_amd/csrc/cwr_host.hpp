@@ -58,13 +58,15 @@ int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                    i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode, int* status,
-                   float* costs_or_null, hipStream_t stream);
+                   float* costs_or_null, float* reduced_or_null, hipStream_t stream);
 // grads (may be null): rows of skipped sequences get a zero record there
 int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads);
 int launch_rowinfo(const Batch& b, int* rowinfo);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
-int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs);
-int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs);
+// reduced (may be null): 2 floats, sum and mean of the N costs
+int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs,
+                float* reduced);
+int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs, float* reduced);
 // d(total) / d(cost of sequence n) = p[n * stride] * scale; stride 0 broadcasts one value
 struct GradOut {
     const float* p;

@@ -72,10 +72,11 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                                                 i64* __restrict__ row_off, i64* __restrict__ lab_off,
                                                 i64* __restrict__ pad_off, i64* __restrict__ slot_off,
                                                 i64* __restrict__ bnd_off, int* __restrict__ seqmode,
-                                                int* __restrict__ status, float* __restrict__ costs) {
+                                                int* __restrict__ status, float* __restrict__ costs,
+                                                float* __restrict__ reduced) {
     const int lane = threadIdx.x;
     i64 carry_r = 0, carry_l = 0, carry_p = 0, carry_b = 0;
-    int flags = 0;
+    int flags = 0, usable = 0;
     for (i64 base = 0; base < N; base += 64) {
         const i64 i = base + lane;
         i64 rows = 0, labs = 0;
@@ -117,6 +118,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                     flags |= CWR_FLAG_U_TOO_LARGE;
                 }
                 pad_off[i] = ok ? ps : -1;
+                usable += ok ? 1 : 0;
                 slot_off[i] = ps;
                 bnd_off[i] = bs;
                 seqmode[i] = 0;
@@ -134,6 +136,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
     flags |= __shfl_xor(flags, 8);
     flags |= __shfl_xor(flags, 16);
     flags |= __shfl_xor(flags, 32);
+    for (int m = 1; m < 64; m <<= 1) usable += __shfl_xor(usable, m);
     if (lane == 0) {
         row_off[N] = carry_r;
         lab_off[N] = carry_l;
@@ -144,17 +147,21 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
         }
         if (R >= 0 && carry_r != R) flags |= CWR_FLAG_ROWS_MISMATCH;
         status[0] = flags;
-        status[1] = 0;
-        status[2] = 0;
+        status[1] = usable;  // sequences whose cost a later kernel writes (the others hold NaN already)
+        status[2] = 0;       // how many of them have been written
         status[3] = 0;
+        if (reduced && usable == 0) {  // no later kernel will write a cost: all of them are NaN
+            reduced[0] = __int_as_float(0x7fc00000);
+            reduced[1] = __int_as_float(0x7fc00000);
+        }
     }
 }
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                    i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode,
-                   int* status, float* costs, hipStream_t stream) {
+                   int* status, float* costs, float* reduced, hipStream_t stream) {
     hipLaunchKernelGGL(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
-                       row_off, lab_off, pad_off, slot_off, bnd_off, seqmode, status, costs);
+                       row_off, lab_off, pad_off, slot_off, bnd_off, seqmode, status, costs, reduced);
     return check_launch();
 }
 
@@ -748,12 +755,36 @@ struct LatticeView {
     }
 };
 
+// Sum and mean of the N costs (cwarp_rnnt/__init__.py:66-71), by the wave that writes the last
+// of them: every writer counts itself in after making its cost visible, and the wave that sees
+// the count complete adds all N up in a fixed order (lane i takes costs i, i+64, ...; then a
+// butterfly), so the result does not depend on which wave came last.  Called by whole waves.
+__device__ __forceinline__ void finish_costs(bool wrote, int N, float* costs, float* reduced, int* status) {
+    if (!reduced) return;
+    bool last = false;
+    if (wrote) {
+        __threadfence();
+        last = atomicAdd(&status[2], 1) == status[1] - 1;
+    }
+    if (__ballot(last) == 0) return;
+    __threadfence();
+    const int lane = threadIdx.x & 63;
+    double s = 0.0;
+    for (int i = lane; i < N; i += 64)
+        s += (double)__hip_atomic_load(&costs[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int m = 1; m < 64; m <<= 1) s += __shfl_xor(s, m);
+    if (lane == 0) {
+        reduced[0] = (float)s;
+        reduced[1] = (float)(s / (double)N);
+    }
+}
+
 // One thread per lattice SLOT, so that a wave reads alpha, beta and the cell records of 64
 // neighbouring slots (consecutive addresses; a thread per compact row would touch one cache line
 // per lane, the strip layout being diagonal to the row order).  The two successors of cell (t,u)
 // sit one strip row further: same column (t+1,u) and next column (t,u+1); only the last column of a
 // strip looks into the next strip.  The 8-byte results are scattered to the row order.
-__global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
+__device__ __forceinline__ bool fill_slot(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
                                                const i64* __restrict__ pad_off,
                                                const i64* __restrict__ slot_off,
@@ -763,6 +794,7 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
                                                const int* __restrict__ scale_a, const int* __restrict__ scale_b,
                                                float2* __restrict__ grads, float* __restrict__ costs,
                                                int* __restrict__ status) {
+    // returns whether this thread wrote its sequence's cost
     const i64 slot = (i64)blockIdx.x * 256 + threadIdx.x;
     // the sequence whose slots hold this one: the last n with slot_off[n] <= slot (skipped
     // sequences have no slots)
@@ -783,9 +815,9 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
                           (unsigned)__builtin_amdgcn_readlane((int)mine, i);
             if (slot >= b) n = i;
         }
-        if (slot >= total) return;
+        if (slot >= total) return false;
     } else {
-        if (slot >= slot_off[N]) return;
+        if (slot >= slot_off[N]) return false;
         int lo = 0, hi = N;
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
@@ -794,7 +826,7 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
         n = lo;
     }
     const i64 pad = pad_off[n];
-    if (pad < 0) return;
+    if (pad < 0) return false;
     const int T = lx[n], U = ly[n];
     const int Up = U + 1;
     const int S = (Up + 63) >> 6;
@@ -807,9 +839,9 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
     const int row = rem / nl;
     const int l = rem - row * nl;
     const int t = row - l - kRowShift, u = (s << 6) + l;
-    if (t < 0 || t >= T) return;  // padding
+    if (t < 0 || t >= T) return false;  // padding
     const i64 r = row_off[n] + (i64)t * Up + u;
-    if (r >= R) return;
+    if (r >= R) return false;
     const int mode = seqmode[n];
     LatticeView A, Bv;
     A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
@@ -841,16 +873,34 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
             fb = (fa + fb) * 0.5;
         }
         costs[n] = (float)(-fb * (double)kLn2);
+        return true;
     }
+    return false;
 }
 
-int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs) {
+__global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
+                                               const i64* __restrict__ row_off,
+                                               const i64* __restrict__ pad_off,
+                                               const i64* __restrict__ slot_off,
+                                               const int* __restrict__ seqmode, int N, i64 R,
+                                               const LpCell* __restrict__ lp,
+                                               const double* __restrict__ alpha, const double* __restrict__ beta,
+                                               const int* __restrict__ scale_a, const int* __restrict__ scale_b,
+                                               float2* __restrict__ grads, float* costs, float* reduced,
+                                               int* status) {
+    const bool wrote = fill_slot(lx, ly, row_off, pad_off, slot_off, seqmode, N, R, lp, alpha, beta, scale_a,
+                                 scale_b, grads, costs, status);
+    finish_costs(wrote, N, costs, reduced, status);
+}
+
+int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs,
+                float* reduced) {
     if (b.R == 0) return CWR_OK;
     const i64 slots = ws.slot_cap;  // the device knows the exact count; threads beyond it leave at once
     if ((slots + 255) / 256 > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
     hipLaunchKernelGGL(k_fill, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
                        ws.pad_off, ws.slot_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
-                       ws.scale_b, reinterpret_cast<float2*>(grads), costs, b.status);
+                       ws.scale_b, reinterpret_cast<float2*>(grads), costs, reduced, b.status);
     (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
     return check_launch();
 }
@@ -859,22 +909,25 @@ __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ l
                                                        const i64* __restrict__ pad_off,
                                                        const int* __restrict__ seqmode, int N,
                                                        const double* __restrict__ beta,
-                                                       const int* __restrict__ scale_b,
-                                                       float* __restrict__ costs) {
+                                                       const int* __restrict__ scale_b, float* costs,
+                                                       float* reduced, int* status) {
     const int n = blockIdx.x * 64 + threadIdx.x;
-    if (n >= N) return;
-    const i64 pad = pad_off[n];
-    if (pad < 0) return;  // NaN already set by k_offsets
-    LatticeView Bv;
-    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
-    Bv.linear = linear_beta(seqmode[n], (Bv.Up + 63) >> 6);
-    costs[n] = (float)(-Bv.log2_at(0, 0) * (double)kLn2);
+    bool wrote = false;
+    const i64 pad = n < N ? pad_off[n] : -1;
+    if (pad >= 0) {  // else: NaN already set by k_offsets
+        LatticeView Bv;
+        Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
+        Bv.linear = linear_beta(seqmode[n], (Bv.Up + 63) >> 6);
+        costs[n] = (float)(-Bv.log2_at(0, 0) * (double)kLn2);
+        wrote = true;
+    }
+    finish_costs(wrote, N, costs, reduced, status);
 }
 
-int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs) {
+int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs, float* reduced) {
     if (b.N == 0) return CWR_OK;
     hipLaunchKernelGGL(k_cost_from_beta, dim3((unsigned)((b.N + 63) / 64)), dim3(64), 0, b.stream, b.lx,
-                       b.ly, ws.pad_off, ws.seqmode, b.N, ws.beta, ws.scale_b, costs);
+                       b.ly, ws.pad_off, ws.seqmode, b.N, ws.beta, ws.scale_b, costs, reduced, b.status);
     return check_launch();
 }
 

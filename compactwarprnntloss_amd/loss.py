@@ -41,7 +41,7 @@ def _label_args(ys: torch.Tensor):
 class ForwardState:
     """What a forward call leaves behind for the backward pass and for inspection."""
     __slots__ = ("row_off", "lab_off", "status", "rowinfo", "lse", "grads", "workspace", "N", "R", "V", "mode",
-                 "max_u")
+                 "max_u", "reduced")
 
 
 def _check_inputs(xs, lx, ys, ly):
@@ -63,8 +63,9 @@ def _check_inputs(xs, lx, ys, ly):
 
 
 def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] = None,
-                 with_grad: bool = True):
-    """Binding of cwr_forward / cwr_loss.  Returns (costs fp32 (N,), ForwardState)."""
+                 with_grad: bool = True, reduce: bool = False):
+    """Binding of cwr_forward / cwr_loss (and their *_reduced forms).  Returns (costs fp32 (N,),
+    ForwardState); with reduce=True the state also holds `reduced` = (sum, mean) of the costs."""
     _check_inputs(xs, lx, ys, ly)
     lib = _lib.load()
     dev = xs.device
@@ -83,7 +84,10 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     st.status = meta[2 * (N + 1):].view(torch.int32)
     ws_bytes = lib.cwr_workspace_bytes(N, R, int(max_u))
     st.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    costs = torch.empty(N, dtype=torch.float32, device=dev)
+    # the costs and, behind them, their sum and mean
+    cbuf = torch.empty(N + 2, dtype=torch.float32, device=dev)
+    costs = cbuf[:N]
+    st.reduced = cbuf[N:] if (reduce and N > 0) else None
     st.lse = torch.empty(R, dtype=torch.float32, device=dev) if (fused and with_grad) else None
     st.grads = torch.empty((R, 2), dtype=torch.float32, device=dev) if with_grad else None
     st.rowinfo = torch.empty((R, 2), dtype=torch.int32, device=dev) if with_grad else None
@@ -93,13 +97,15 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
                   y_stride, y_len, N, int(blank), mode, int(max_u),
                   st.workspace.data_ptr(), ws_bytes, st.row_off.data_ptr(), st.lab_off.data_ptr(),
                   st.status.data_ptr())
+        red = (st.reduced.data_ptr(),) if st.reduced is not None else ()
         if with_grad:
-            rc = lib.cwr_forward(*common, st.rowinfo.data_ptr(),
-                                 st.lse.data_ptr() if st.lse is not None else None,
-                                 st.grads.data_ptr(), costs.data_ptr(), _stream_ptr(dev))
+            fn = lib.cwr_forward_reduced if red else lib.cwr_forward
+            rc = fn(*common, st.rowinfo.data_ptr(), st.lse.data_ptr() if st.lse is not None else None,
+                    st.grads.data_ptr(), costs.data_ptr(), *red, _stream_ptr(dev))
             _lib.check(rc, "cwr_forward")
         else:
-            rc = lib.cwr_loss(*common, costs.data_ptr(), _stream_ptr(dev))
+            fn = lib.cwr_loss_reduced if red else lib.cwr_loss
+            rc = fn(*common, costs.data_ptr(), *red, _stream_ptr(dev))
             _lib.check(rc, "cwr_loss")
     return costs, st
 
@@ -242,7 +248,8 @@ class _TransLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx: Any, xs, lx, ys, ly, blank, fused, max_u, validate, reduction, fastemit_lambda=0.0):
         need_grad = xs.requires_grad
-        costs, st = rnnt_forward(xs, lx, ys, ly, blank, fused, max_u, with_grad=need_grad)
+        costs, st = rnnt_forward(xs, lx, ys, ly, blank, fused, max_u, with_grad=need_grad,
+                                 reduce=reduction in ("mean", "sum"))
         if validate:
             _raise_on_flags(st)
         if need_grad:
@@ -253,8 +260,10 @@ class _TransLoss(torch.autograd.Function):
             ctx.blank = blank
             ctx.reduction = reduction
             ctx.save_for_backward(xs, lx, ys, ly)
-        if xs.dtype not in (torch.float16, torch.bfloat16):
-            costs = costs.to(xs.dtype)
+        out_dtype = xs.dtype if xs.dtype not in (torch.float16, torch.bfloat16) else torch.float32
+        if st.reduced is not None:  # summed on the device by the kernel that wrote the last cost
+            return st.reduced[1 if reduction == "mean" else 0].to(out_dtype)
+        costs = costs.to(out_dtype)
         if reduction == "mean":
             return costs.mean()
         if reduction == "sum":

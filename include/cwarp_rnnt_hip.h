@@ -115,7 +115,8 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R,
  *   max_u    an upper bound of max(ly) known to the host (e.g. the padded label width); a
  *            sequence with more labels is skipped (cost NaN, CWR_FLAG_U_TOO_LARGE)
  * outputs
- *   row_off, lab_off (N+1) int64;  status 4 x int32
+ *   row_off, lab_off (N+1) int64;  status 4 x int32 (word 0: CWR_FLAG_* bits; the others are
+ *            scratch of the call)
  *   rowinfo  (R,2) int32 per-row record for cwr_backward: (label of the row or -1, sequence of the
  *            row or -1)
  *   lse      (R,) fp32 log-sum-exp of each row            [CWR_MODE_FUSED only, else may be NULL]
@@ -137,6 +138,23 @@ int cwr_loss(const void* x, int dtype, int64_t R, int64_t V,
              void* workspace, size_t workspace_bytes,
              int64_t* row_off, int64_t* lab_off, int32_t* status,
              float* costs, void* stream);
+
+/* cwr_forward / cwr_loss with the reduction of cwarp_rnnt/__init__.py:66-71 folded in: besides
+ * costs, reduced[0] = sum of the N costs and reduced[1] = their mean (2 x fp32), written by
+ * whichever wave writes the last cost and summed in a fixed order, so that 'mean' / 'sum' need no
+ * further kernel.  A skipped sequence (cost NaN) makes both NaN.  N = 0 writes nothing. */
+int cwr_forward_reduced(const void* x, int dtype, int64_t R, int64_t V,
+                        const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                        int64_t N, int32_t blank, int mode, int64_t max_u,
+                        void* workspace, size_t workspace_bytes,
+                        int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
+                        float* lse, float* grads, float* costs, float* reduced, void* stream);
+int cwr_loss_reduced(const void* x, int dtype, int64_t R, int64_t V,
+                     const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                     int64_t N, int32_t blank, int mode, int64_t max_u,
+                     void* workspace, size_t workspace_bytes,
+                     int64_t* row_off, int64_t* lab_off, int32_t* status,
+                     float* costs, float* reduced, void* stream);
 
 /* Gradient w.r.t. x.  Replaces _cwarp_rnnt_backward (cwarp_cuda.cpp:110-136 ->
  * cwarp_cuda_backward_ + zeros(R,V) + gather_cuda_backward_) in one streaming pass that does

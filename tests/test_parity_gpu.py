@@ -485,3 +485,44 @@ def test_uniform_lattice_of_tiny_probabilities_matches_the_closed_form():
     np.testing.assert_allclose(dev["costs"], want, rtol=LOSS_RTOL)
     ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "logprob")
     np.testing.assert_allclose(dev["G"], ref["G"], rtol=0, atol=GRAD_ATOL)
+
+
+@pytest.mark.parametrize("with_grad", [True, False])
+@pytest.mark.parametrize("N", [1, 5, 64, 150])
+def test_reduction_folded_into_the_forward_call(with_grad, N):
+    """cwr_forward_reduced / cwr_loss_reduced: sum and mean of the costs come out of the call that
+    computes them (cwarp_rnnt/__init__.py:66-71), identical from run to run."""
+    pkg = _pkg()
+    rng = np.random.default_rng(N)
+    b = make_batch(rng.integers(1, 20, N), rng.integers(0, 9, N), 12, seed=N)
+    dev = torch.device("cuda:0")
+    xs = b["x"].to(dev)
+    lx, ly = torch.from_numpy(b["lx"]).to(dev), torch.from_numpy(b["ly"]).to(dev)
+    ys = torch.from_numpy(b["yp"]).to(dev)
+    seen = set()
+    for _ in range(3):
+        costs, st = pkg.rnnt_forward(xs, lx, ys, ly, 0, True, with_grad=with_grad, reduce=True)
+        red = st.reduced.cpu().numpy()
+        c = costs.double().cpu().numpy()
+        np.testing.assert_allclose(red[0], c.sum(), rtol=1e-6)
+        np.testing.assert_allclose(red[1], c.mean(), rtol=1e-6)
+        seen.add((float(red[0]), float(red[1])))
+    assert len(seen) == 1
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "fused", want_dense=False)
+    np.testing.assert_allclose(red[1], ref["costs"].mean(), rtol=LOSS_RTOL)
+
+
+def test_reduction_is_nan_when_a_sequence_is_skipped():
+    pkg = _pkg()
+    b = make_batch([6, 4, 9], [2, 3, 1], 10, seed=2)
+    dev = torch.device("cuda:0")
+    xs = b["x"].to(dev)
+    lx = torch.tensor([6, 0, 9], dtype=torch.int32, device=dev)       # a sequence without frames
+    ly = torch.from_numpy(b["ly"]).to(dev)
+    ys = torch.from_numpy(b["yp"]).to(dev)
+    costs, st = pkg.rnnt_forward(xs, lx, ys, ly, 0, True, reduce=True)
+    assert int(st.status[0].item()) & 2
+    assert torch.isnan(costs[1]) and torch.isnan(st.reduced).all()
+    lx0 = torch.zeros(3, dtype=torch.int32, device=dev)                # nothing usable at all
+    costs, st = pkg.rnnt_forward(xs, lx0, ys, ly, 0, True, reduce=True)
+    assert torch.isnan(costs).all() and torch.isnan(st.reduced).all()
