@@ -400,6 +400,114 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     }
 }
 
+// Long rows, and rows that do not start on a 16-byte boundary (V not a multiple of VEC): one wave
+// per row, walking the 16-byte packs that cover it in chunks of 64*KC, the next chunk's loads in
+// flight while the current one is reduced.  Every lane keeps a running (max, sum of exponentials)
+// of its own elements, rescaled once per chunk, and the lanes are merged once at the end.  The
+// packs at either end of an unaligned row also hold elements of the neighbouring rows: those are
+// masked.  The tensor's first and last pack are whole (its base is 16-byte aligned and only packs
+// that lie inside it are read: a ragged tail is read element by element).
+template <typename T, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
+    const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
+    const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int KC = 4;
+    const int lane = threadIdx.x & 63;
+    const i64 r = wave_first_row<true>(1);
+    if (r >= R) return;
+    const i64 e0 = r * (i64)V, e1 = e0 + V;        // the row's elements in the flat tensor
+    const i64 total = R * (i64)V;
+    const i64 p0 = e0 / VEC;                       // first pack that holds any of them
+    const i64 p_end = (e1 + VEC - 1) / VEC;        // one past the last
+    const i64 p_whole = total / VEC;               // packs that lie inside the tensor
+    const int P = (int)(p_end - p0);
+    const T* row = x + e0;
+
+    auto fetch = [&](int chunk, v4i (&raw)[KC]) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const i64 p = p0 + (i64)chunk * (64 * KC) + k * 64 + lane;
+            raw[k] = load_raw<NT>(x + (p < p_end && p < p_whole ? p : p0) * VEC);
+        }
+    };
+    v4i buf_a[KC], buf_b[KC];
+    fetch(0, buf_a);
+    // the row's place in the batch, while the first loads are in flight
+    int lab = -1;
+    i64 dst = -1;
+    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+    const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+    if (pad >= 0) {
+        lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+        dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+    }
+    const float xb = Elem<T>::to_f32(row[blank]);
+    const float xl = Elem<T>::to_f32(row[lab < 0 ? 0 : lab]);
+
+    float m = -INFINITY, s = 0.f;  // this lane's running maximum and sum of 2^((x - m) log2 e)
+    auto reduce = [&](int ch, const v4i (&raw)[KC]) {
+        float xv[KC][VEC];
+        float cm = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < KC; ++k) {
+            const i64 p = p0 + (i64)ch * (64 * KC) + k * 64 + lane;
+            Pack<T>::unpack(raw[k], xv[k]);
+            // components [lo, hi) of this pack belong to the row: all of them, except in the packs at
+            // its two ends, and none in a pack beyond it
+            int lo = 0, hi = (p < p_end && p < p_whole) ? VEC : 0;
+            if (p == p0) lo = (int)(e0 - p * VEC);
+            if (p + 1 >= p_end && hi) hi = (int)(e1 - p * VEC) < VEC ? (int)(e1 - p * VEC) : VEC;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                xv[k][c] = (c >= lo && c < hi) ? xv[k][c] : -INFINITY;
+                cm = fmaxf(cm, xv[k][c]);
+            }
+        }
+        if (cm > m) {  // rescale what has been summed so far (m = -inf: s = 0 stays 0)
+            s *= fast_exp2((m - cm) * kLog2e);
+            m = cm;
+        }
+        if (m > -INFINITY) {
+            const float ms = m * kLog2e;
+#pragma unroll
+            for (int k = 0; k < KC; ++k)
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) s += fast_exp2(fmaf(xv[k][c], kLog2e, -ms));
+        }
+    };
+    // two buffers taking turns, so that no register with a load in flight is ever copied
+    const int chunks = (P + 64 * KC - 1) / (64 * KC);
+    for (int ch = 0; ch < chunks; ch += 2) {
+        if (ch + 1 < chunks) fetch(ch + 1, buf_b);
+        reduce(ch, buf_a);
+        if (ch + 1 < chunks) {
+            if (ch + 2 < chunks) fetch(ch + 2, buf_a);
+            reduce(ch + 1, buf_b);
+        }
+    }
+    // a ragged end of the tensor (its last, partial pack) belongs to the last row: element by element
+    if (p_end > p_whole && lane == 0) {
+        for (i64 e = p_whole * VEC < e0 ? e0 : p_whole * VEC; e < e1; ++e) {
+            const float v = Elem<T>::to_f32(x[e]);
+            if (v > m) { s *= fast_exp2((m - v) * kLog2e); m = v; }
+            s += fast_exp2((v - m) * kLog2e);
+        }
+    }
+    const float M = group_allreduce<64, OpMax>(m);
+    const float S = group_allreduce<64, OpSum>(m > -INFINITY ? s * fast_exp2((m - M) * kLog2e) : 0.f);
+    const float lse = fmaf(fast_log2(S), kLn2, M);
+    if (lane == 0) {
+        lse_out[r] = lse;
+        rowinfo[r] = make_int2(lab, ri.n);
+        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
+    }
+}
+
 // Any V, any alignment: one wave per row, scalar accesses.
 template <typename T>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
@@ -518,6 +626,86 @@ __device__ __forceinline__ v4i grad_pack(v4i in, const RowCoef& rc, int pack, in
     return Pack<T>::pack(o);
 }
 
+// The VEC gradient values of a pack whose first element is column v0 of a row with coefficients rc
+// (v0 may be negative or beyond V for the part of a pack that belongs to a neighbouring row: the
+// blank / label positions then simply do not occur in it).
+template <typename T, bool FUSED>
+__device__ __forceinline__ void grad_elems(const float (&xv)[Elem<T>::VEC], const RowCoef& rc, int v0, int blank,
+                                           float (&o)[Elem<T>::VEC]) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int cb_at = blank - v0;
+    const int cl_at = rc.lab >= 0 ? rc.lab - v0 : -1;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) {
+        float v = FUSED ? fast_exp2(fmaf(xv[c], kLog2e, rc.nls)) * rc.cg : 0.f;
+        if (FUSED) {
+            v += c == cb_at ? rc.cb : 0.f;
+            v += c == cl_at ? rc.cl : 0.f;
+        } else {
+            v = c == cb_at ? rc.cb : v;
+            v = c == cl_at ? rc.cl : v;  // label after blank, as the reference's scatter
+        }
+        o[c] = v;
+    }
+}
+
+// Any V of at least 64*VEC, aligned or not: the (R,V) tensor is walked as one flat array of 16-byte
+// packs, 64 per wave, whatever the rows do.  A wave then touches at most two rows (their
+// coefficients come through the scalar unit) and at most one of its packs straddles them.
+template <typename T, bool FUSED, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_any(
+    const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
+    const float2* __restrict__ grads, const float* __restrict__ lse, const GradOut grad_costs,
+    T* __restrict__ gx) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const i64 wave = wave_first_row<true>(1);  // global wave index
+    const i64 total = R * (i64)V;
+    const i64 E0 = wave * (64 * VEC);
+    if (E0 >= total) return;
+    const i64 ra = E0 / V;
+    const i64 a_start = ra * V, b_start = a_start + V;  // row ra, and the row after it
+    const bool two = b_start < E0 + 64 * VEC && ra + 1 < R;
+    const RowCoef ca = row_coef<FUSED>(ra, N, rowinfo, grads, lse, grad_costs);
+    const RowCoef cb = two ? row_coef<FUSED>(ra + 1, N, rowinfo, grads, lse, grad_costs) : ca;
+    const i64 e = E0 + (i64)lane * VEC;
+    if (e >= total) return;
+    float xv[VEC], o[VEC];
+    if (e + VEC <= total) {
+        if (FUSED) Pack<T>::unpack(load_raw<NT>(x + e), xv);
+        const bool in_b = e >= b_start;
+        const bool straddle = !in_b && e + VEC > b_start;
+        RowCoef rc;
+        rc.cg = in_b ? cb.cg : ca.cg; rc.cb = in_b ? cb.cb : ca.cb; rc.cl = in_b ? cb.cl : ca.cl;
+        rc.nls = in_b ? cb.nls : ca.nls; rc.lab = in_b ? cb.lab : ca.lab;
+        grad_elems<T, FUSED>(xv, rc, (int)(e - (in_b ? b_start : a_start)), blank, o);
+        if (straddle) {
+            float ob[VEC];
+            grad_elems<T, FUSED>(xv, cb, (int)(e - b_start), blank, ob);
+            const int split = (int)(b_start - e);
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) o[c] = c >= split ? ob[c] : o[c];
+        }
+        store_raw<NT>(gx + e, Pack<T>::pack(o));
+    } else {
+        // the tensor's ragged tail (fewer than VEC elements): element by element
+        for (i64 g = e; g < total; ++g) {
+            const bool in_b = g >= b_start;
+            const RowCoef& rc = in_b ? cb : ca;
+            const int v = (int)(g - (in_b ? b_start : a_start));
+            float val = FUSED ? fast_exp2(fmaf(Elem<T>::to_f32(x[g]), kLog2e, rc.nls)) * rc.cg : 0.f;
+            if (FUSED) {
+                val += v == blank ? rc.cb : 0.f;
+                val += v == rc.lab ? rc.cl : 0.f;
+            } else {
+                val = v == blank ? rc.cb : val;
+                val = v == rc.lab ? rc.cl : val;
+            }
+            gx[g] = Elem<T>::from_f32(val);
+        }
+    }
+}
+
 // Rows of NV = 64*CH packs: a wave moves 64 consecutive packs of one row, one per lane.  The row
 // is wave-uniform, so its coefficients come through the scalar unit.
 template <typename T, bool FUSED, bool NT>
@@ -631,6 +819,8 @@ static bool pick_shape(int NV, int* lpr, int* k) {
     return false;
 }
 
+static bool base_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 template <typename T>
 static bool packed_ok(const void* p, int V) {
     return V % Elem<T>::VEC == 0 && (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
@@ -683,6 +873,13 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
 #undef CWR_ROWS
 #undef CWR_ARGS
     }
+    if (base_aligned(b.x) && b.V >= 64 * Elem<T>::VEC) {  // long rows, or rows off the 16-byte grid
+        hipLaunchKernelGGL((k_gather_long<T, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u),
+                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride,
+                           b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode,
+                           b.status);
+        return check_launch();
+    }
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
                        ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);
@@ -719,6 +916,14 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
             CWR_SHAPES(CWR_CASE)
 #undef CWR_CASE
         }
+    }
+    if (base_aligned(grad_x) && (!FUSED || base_aligned(b.x)) && b.V >= 64 * Elem<T>::VEC) {
+        const i64 per_wave = 64 * Elem<T>::VEC;
+        const i64 waves = (b.R * (i64)b.V + per_wave - 1) / per_wave;
+        hipLaunchKernelGGL((k_grad_any<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
+                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse,
+                           grad_costs, gx);
+        return check_launch();
     }
     hipLaunchKernelGGL((k_grad_generic<T, FUSED>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64), 0,
                        b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);
