@@ -508,6 +508,56 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
     }
 }
 
+// Short rows of any length and alignment (V below 64 packs, where the packed kernels do not
+// apply: V not a multiple of the pack, or an unaligned tensor): LPR lanes per row, element-wise
+// loads all issued up front, 64/LPR rows per wave.
+template <typename T, int LPR, int KMAX>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_small(
+    const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
+    const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
+    const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
+    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
+    constexpr int RP = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int g = lane / LPR, j = lane - g * LPR;
+    const i64 r = wave_first_row(RP) + g;
+    const bool live = r < R;
+    const T* row = x + (live ? r : 0) * (i64)V;
+    float xv[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        const int v = j + k * LPR;
+        xv[k] = (live && v < V) ? Elem<T>::to_f32(row[v]) : -INFINITY;
+    }
+    float m = xv[0];
+#pragma unroll
+    for (int k = 1; k < KMAX; ++k) m = fmaxf(m, xv[k]);
+    m = group_allreduce<LPR, OpMax>(m);
+    const float ms = m * kLog2e;
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) s += fast_exp2(fmaf(xv[k], kLog2e, -ms));
+    s = group_allreduce<LPR, OpSum>(s);
+    const float lse = fmaf(fast_log2(s), kLn2, m);
+    if (live && j == 0) {
+        lse_out[r] = lse;
+        const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+        int lab = -1;
+        if (pad >= 0) {
+            lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+            const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
+            const float xb = Elem<T>::to_f32(row[blank]);
+            const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
+            lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        } else if (grads_skipped) {
+            grads_skipped[r] = make_float2(0.f, 0.f);
+        }
+        rowinfo[r] = make_int2(lab, ri.n);
+    }
+}
+
 // Any V, any alignment: one wave per row, scalar accesses.
 template <typename T>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
@@ -706,6 +756,63 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_any(
     }
 }
 
+// Short rows (VEC <= V < 64 packs) of any length: the same flat walk, but a wave now covers many
+// rows, so every lane finds the (at most two) rows of its pack and fetches their coefficients
+// itself.
+template <typename T, bool FUSED, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_small(
+    const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
+    const float2* __restrict__ grads, const float* __restrict__ lse, const GradOut grad_costs,
+    T* __restrict__ gx) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const i64 wave = wave_first_row<true>(1);
+    const i64 total = R * (i64)V;
+    const i64 E0 = wave * (64 * VEC);
+    if (E0 >= total) return;
+    const i64 r0 = E0 / V;                                  // wave-uniform: one 64-bit division per wave
+    const unsigned in0 = (unsigned)(E0 - r0 * V) + (unsigned)lane * VEC;
+    const unsigned dr = in0 / (unsigned)V;
+    const i64 ra = r0 + dr;
+    const int v0 = (int)(in0 - dr * (unsigned)V);           // column of the pack's first element in row ra
+    const i64 e = E0 + (i64)lane * VEC;
+    if (e >= total) return;
+    const bool two = v0 + VEC > V && ra + 1 < R;            // V >= VEC: a pack meets at most two rows
+    float xv[VEC], o[VEC];
+    const bool whole = e + VEC <= total;
+    if (FUSED && whole) Pack<T>::unpack(load_raw<NT>(x + e), xv);
+    // both rows' coefficients are fetched by every lane (neighbouring lanes share them, and a
+    // branch around the second fetch would put its latency behind the first one's)
+    const RowCoef ca = row_coef<FUSED>(ra, N, rowinfo, grads, lse, grad_costs);
+    const RowCoef cb = row_coef<FUSED>(ra + 1 < R ? ra + 1 : ra, N, rowinfo, grads, lse, grad_costs);
+    if (whole) {
+        grad_elems<T, FUSED>(xv, ca, v0, blank, o);
+        if (two) {
+            float ob[VEC];
+            grad_elems<T, FUSED>(xv, cb, v0 - V, blank, ob);
+            const int split = V - v0;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) o[c] = c >= split ? ob[c] : o[c];
+        }
+        store_raw<NT>(gx + e, Pack<T>::pack(o));
+    } else {
+        for (i64 g = e; g < total; ++g) {  // the tensor's ragged tail
+            const i64 rr = g / V;
+            const int v = (int)(g - rr * V);
+            const RowCoef rc = row_coef<FUSED>(rr, N, rowinfo, grads, lse, grad_costs);
+            float val = FUSED ? fast_exp2(fmaf(Elem<T>::to_f32(x[g]), kLog2e, rc.nls)) * rc.cg : 0.f;
+            if (FUSED) {
+                val += v == blank ? rc.cb : 0.f;
+                val += v == rc.lab ? rc.cl : 0.f;
+            } else {
+                val = v == blank ? rc.cb : val;
+                val = v == rc.lab ? rc.cl : val;
+            }
+            gx[g] = Elem<T>::from_f32(val);
+        }
+    }
+}
+
 // Rows of NV = 64*CH packs: a wave moves 64 consecutive packs of one row, one per lane.  The row
 // is wave-uniform, so its coefficients come through the scalar unit.
 template <typename T, bool FUSED, bool NT>
@@ -880,6 +987,18 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
                            b.status);
         return check_launch();
     }
+    if (b.V < 64 * Elem<T>::VEC) {  // short rows off the packed paths
+#define CWR_SMALL(L, KM)                                                                             \
+    if (b.V <= L * KM) {                                                                             \
+        hipLaunchKernelGGL((k_gather_small<T, L, KM>), dim3(blocks_for_waves((b.R + 64 / L - 1) / (64 / L))), \
+                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, \
+                           b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz,     \
+                           ws.seqmode, b.status);                                                    \
+        return check_launch();                                                                       \
+    }
+        CWR_SMALL(8, 4) CWR_SMALL(8, 8) CWR_SMALL(16, 8) CWR_SMALL(32, 8) CWR_SMALL(64, 8)
+#undef CWR_SMALL
+    }
     hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
                        ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);
@@ -921,6 +1040,14 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
         const i64 per_wave = 64 * Elem<T>::VEC;
         const i64 waves = (b.R * (i64)b.V + per_wave - 1) / per_wave;
         hipLaunchKernelGGL((k_grad_any<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
+                           dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse,
+                           grad_costs, gx);
+        return check_launch();
+    }
+    if (base_aligned(grad_x) && (!FUSED || base_aligned(b.x)) && b.V >= Elem<T>::VEC) {
+        const i64 per_wave = 64 * Elem<T>::VEC;
+        const i64 waves = (b.R * (i64)b.V + per_wave - 1) / per_wave;
+        hipLaunchKernelGGL((k_grad_small<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
                            dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse,
                            grad_costs, gx);
         return check_launch();
