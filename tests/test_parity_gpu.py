@@ -529,3 +529,32 @@ def test_reduction_is_nan_when_a_sequence_is_skipped():
     lx0 = torch.zeros(3, dtype=torch.int32, device=dev)                # nothing usable at all
     costs, st = pkg.rnnt_forward(xs, lx0, ys, ly, 0, True, reduce=True)
     assert torch.isnan(costs).all() and torch.isnan(st.reduced).all()
+
+
+# ----------------------------------------------------------------------------- randomised sweep
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_against_oracle(seed):
+    """Twenty random batches per seed: sizes, vocabularies (aligned or not), storage types, modes,
+    blank positions, label layouts and logit scales drawn together, so that combinations no
+    hand-written case lists still meet the oracle."""
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(20):
+        N = int(rng.integers(1, 9))
+        big_u = rng.random() < 0.15
+        lx = rng.integers(1, 40, N)
+        ly = rng.integers(0, 200 if big_u else 30, N)
+        V = int(rng.choice([2, 3, 7, 16, 29, 41, 64, 96, 130, 255, 256, 300, 511, 1024, 1031, 2048, 4099]))
+        if (lx * (ly + 1)).sum() * V > 6e6:
+            V = int(rng.choice([7, 16, 41, 64]))
+        dtype = str(rng.choice(["f32", "f32", "f32", "f16", "bf16", "f64"]))
+        fused = bool(rng.integers(0, 2))
+        blank = int(rng.integers(0, V))
+        sigma = float(rng.choice([0.5, 1.0, 2.0, 6.0]))
+        labels = str(rng.choice(["2d", "1d"]))
+        b = make_batch(lx, ly, V, seed=int(rng.integers(1 << 30)), sigma=sigma, dtype=dtype, blank=blank,
+                       normalised=not fused)
+        try:
+            check_case(b, fused, labels, dtype=dtype, seed=case)
+        except AssertionError as err:
+            raise AssertionError(f"seed {seed} case {case}: N={N} lx={lx.tolist()} ly={ly.tolist()} V={V} "
+                                 f"{dtype} fused={fused} blank={blank} sigma={sigma} labels={labels}\n{err}")
