@@ -45,6 +45,11 @@ __device__ __forceinline__ float dpp_f32(float old, float src) {
     return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(src),
                                                       CTRL, ROW_MASK, BANK_MASK, false));
 }
+// Lanes without a valid source return 0 (no register has to be cleared first).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32_or_zero(float src) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(src), CTRL, 0xF, 0xF, true));
+}
 template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
 __device__ __forceinline__ int dpp_i32(int old, int src) {
     return __builtin_amdgcn_update_dpp(old, src, CTRL, ROW_MASK, BANK_MASK, false);

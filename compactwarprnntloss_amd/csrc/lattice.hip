@@ -363,7 +363,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     // alpha applies its own cell's probabilities; beta B(t-1,u) and L(t,u-1), the latter from the
     // lane on its left (lane 0 gets 0: nobody reads its `pass`)
     double mul_own = (double)ring[0].x;
-    double mul_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, ring[0].y) : ring[0].y);
+    double mul_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].y) : ring[0].y);
     const double in_mask = lane == in_lane ? 1.0 : 0.0;
     unsigned lo_seen = 0xffffffffu, hi_seen = 0u;  // extremes of the cell values' high words (zero excluded)
     // beta hands on plain beta(t,u+1); the receiving edge column applies its own L(t,u), fetched
@@ -457,7 +457,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = make_double2(BETA ? a : pass, Cd);
             const float2 nx = ring[(j + 1) % kPF];
             mul_own = (double)nx.x;
-            mul_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, nx.y) : nx.y);
+            mul_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.y) : nx.y);
             ring[j] = cn;
             qi += dq;
             mi += dq;
@@ -517,7 +517,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     double pass = kNeg;
     double nbr = kNeg;
     double add_own = (double)ring[0].x;
-    double add_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, ring[0].y) : ring[0].y);
+    double add_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].y) : ring[0].y);
     const int jl = lane & (kPF - 1);
     float edge = 0.f;      // beta: L(t,u) of the edge column's own cells, one block ahead
     double e_next = kNeg;  // global stream: the entries of the next block
@@ -566,7 +566,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
             }
             const float2 nx = ring[(j + 1) % kPF];
             add_own = (double)nx.x;
-            add_pass = (double)(BETA ? dpp_f32<DPP_WAVE_SHR1>(0.f, nx.y) : nx.y);
+            add_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.y) : nx.y);
             ring[j] = cn;
             qi += dq;
             mi += dq;
