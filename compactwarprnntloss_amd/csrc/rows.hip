@@ -174,13 +174,15 @@ __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, co
     float m = xv[0];
 #pragma unroll
     for (int j = 1; j < K * VEC; ++j) m = fmaxf(m, xv[j]);
-    m = group_allreduce<LPR, OpMax>(m);
-    const float ms = m * kLog2e;
-    float s = 0.f;
+    {
+        m = group_allreduce<LPR, OpMax>(m);
+        const float ms = m * kLog2e;
+        float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < K * VEC; ++j) s += fast_exp2(fmaf(xv[j], kLog2e, -ms));
-    s = group_allreduce<LPR, OpSum>(s);
-    lse = fmaf(fast_log2(s), kLn2, m);
+        for (int j = 0; j < K * VEC; ++j) s += fast_exp2(fmaf(xv[j], kLog2e, -ms));
+        s = group_allreduce<LPR, OpSum>(s);
+        lse = fmaf(fast_log2(s), kLn2, m);
+    }
     if (!EXTRACT) return;
     // pick the blank and label entries out of the registers
     const ColPos<VEC, LPR> pl(lab < 0 ? 0 : lab);
@@ -191,15 +193,29 @@ __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, co
         xb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cb), pb.lane));
         xl = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(cl), pl.lane));
     } else {
-        cb = xv[0];
-        cl = xv[0];
+        // the blank sits in the same register and the same lane of every group: scalar reads
+        cb = xv[pb.k * VEC + pb.c];
+        xb = 0.f;
 #pragma unroll
-        for (int c = 1; c < VEC; ++c) {  // K == 1 here
-            cb = c == pb.c ? xv[c] : cb;
-            cl = c == pl.c ? xv[c] : cl;
+        for (int gg = 0; gg < 64 / LPR; ++gg) {
+            const float v = readlane_f32(cb, gg * LPR + pb.lane);
+            xb = gg == g ? v : xb;
         }
-        xb = __shfl(cb, g * LPR + pb.lane);
-        xl = __shfl(cl, g * LPR + pl.lane);
+        if (K == 1) {  // the label's place differs between the groups: select, then one cross-lane read
+            cl = xv[0];
+#pragma unroll
+            for (int c = 1; c < VEC; ++c) cl = c == pl.c ? xv[c] : cl;
+            xl = __shfl(cl, g * LPR + pl.lane);
+        } else {  // group by group, each with wave-uniform positions
+            xl = 0.f;
+#pragma unroll
+            for (int gg = 0; gg < 64 / LPR; ++gg) {
+                const int lab_g = __builtin_amdgcn_readlane(lab, gg * LPR);
+                const ColPos<VEC, LPR> pg(lab_g < 0 ? 0 : lab_g);
+                const float v = readlane_f32(xv[pg.k * VEC + pg.c], gg * LPR + pg.lane);
+                xl = gg == g ? v : xl;
+            }
+        }
     }
 }
 
@@ -289,8 +305,8 @@ __device__ __forceinline__ i64 shfl_i64(i64 v, int src) {
     return ((i64)hi << 32) | (i64)(unsigned)lo;
 }
 
-// Smaller rows: a wave takes NP passes of 64/LPR rows (about 4 KiB in all), issues every load up
-// front, and lane i decodes row r0+i meanwhile.
+// Smaller rows: a wave takes NP passes of 64/LPR rows (4 to 8 KiB in all), issues every load up
+// front, and decodes the rows meanwhile, one row per lane.
 template <typename T, int LPR, int K, int NP, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
@@ -320,9 +336,11 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         }
     }
 
-    // lane i decodes row r0+i
-    const i64 r = r0 + lane;
-    const bool mine = lane < ROWS && r < R;
+    // Lane p of group g decodes the row that group g reduces in pass p, and keeps its results: no
+    // value has to travel between lanes afterwards.
+    static_assert(NP <= LPR && NP <= 16, "one lane of a group per pass");
+    const i64 r = r0 + (i64)lir * RP + g;
+    const bool mine = lir < NP && r < R;
     RowInfo ri;
     ri.n = -1; ri.t = 0; ri.u = 0; ri.T = 0; ri.U = 0; ri.off = 0;
     i64 pad = -1, labbase = 0;
@@ -373,21 +391,24 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     }
 
     const ColPos<VEC, LPR> pb(blank);
-    float res_lse = 0.f, res_b = 0.f, res_l = 0.f;  // results of row r0+i, parked in lane i
+    float res_lse = 0.f, res_b = 0.f, res_l = 0.f;  // results of the lane's own row
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const bool ok = r0 + p * RP + g < R;
 #pragma unroll
         for (int k = 0; k < K; ++k)
             if (!(ok && lir + k * LPR < NV)) raw[p][k] = Pack<T>::neg_inf();
-        const int lab = __shfl(my_lab, p * RP + g);
+        // the label of the row of this pass, from the lane that decoded it
+        int lab;
+        if (RP <= 2) {
+            lab = __builtin_amdgcn_readlane(my_lab, p);
+            if (RP == 2) lab = g == 0 ? lab : __builtin_amdgcn_readlane(my_lab, LPR + p);
+        } else {
+            lab = __shfl(my_lab, g * LPR + p);
+        }
         float lse, xb, xl;
         gather_pass<T, LPR, K>(raw[p], g, pb, lab, lse, xb, xl);
-        const int src = (lane % RP) * LPR;  // lane i = p*RP + j wants the row of group j
-        lse = __shfl(lse, src);
-        xb = __shfl(xb, src);
-        xl = __shfl(xl, src);
-        const bool here = lane / RP == p;
+        const bool here = lir == p;
         res_lse = here ? lse : res_lse;
         res_b = here ? xb : res_b;
         res_l = here ? xl : res_l;
@@ -926,6 +947,19 @@ static bool pick_shape(int NV, int* lpr, int* k) {
     return false;
 }
 
+// The same for the gather pass.  Rows below 4 KiB share a wave: few lanes per row with 4 packs each
+// keep the cross-lane part of the reduction short, and 8 KiB of loads in flight per wave (4 KiB
+// for the shortest rows, whose per-row outputs weigh as much as the row) measured best.
+static bool pick_gather_shape(int NV, int* lpr, int* k) {
+    if (NV < 8) return false;
+    if (NV <= 8) { *lpr = 8; *k = 1; return true; }
+    if (NV <= 16) { *lpr = 16; *k = 1; return true; }
+    if (NV <= 32) { *lpr = 8; *k = 4; return true; }
+    if (NV <= 64) { *lpr = 16; *k = 4; return true; }
+    if (NV <= 128) { *lpr = 32; *k = 4; return true; }
+    return pick_shape(NV, lpr, k);
+}
+
 static bool base_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <typename T>
@@ -956,7 +990,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
         return check_launch();
     }
     int lpr = 0, k = 0;
-    if (packed_ok<T>(b.x, b.V) && pick_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
+    if (packed_ok<T>(b.x, b.V) && pick_gather_shape(b.V / Elem<T>::VEC, &lpr, &k)) {
 #define CWR_ARGS x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,   \
                  b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status
         // grids are multiples of 8 workgroups, see logical_block
@@ -975,7 +1009,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
         return check_launch();                                                                       \
     }
         CWR_ROW(4) CWR_ROW(8) CWR_ROW(16)
-        CWR_ROWS(8, 1, 4) CWR_ROWS(16, 1, 4) CWR_ROWS(32, 1, 4) CWR_ROWS(64, 1, 4) CWR_ROWS(64, 2, 2)
+        CWR_ROWS(8, 1, 8) CWR_ROWS(16, 1, 8) CWR_ROWS(8, 4, 2) CWR_ROWS(16, 4, 2) CWR_ROWS(32, 4, 2)
 #undef CWR_ROW
 #undef CWR_ROWS
 #undef CWR_ARGS

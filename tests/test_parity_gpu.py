@@ -141,7 +141,7 @@ def test_ragged_mix_with_empty_label_and_single_frame(fused):
     check_case(b, fused, "1d")
 
 
-@pytest.mark.parametrize("V", [3, 5, 32, 33, 64, 100, 128, 256, 257, 300, 500, 512, 1000, 1024, 2048, 4096, 4100, 4233,
+@pytest.mark.parametrize("V", [3, 5, 32, 33, 64, 96, 100, 128, 200, 256, 257, 300, 500, 512, 1000, 1024, 2048, 4096, 4100, 4233,
                                5537, 8192, 16384, 32000, 50257])
 def test_vocabulary_sizes_fused(V):
     b = make_batch([6, 3, 9], [2, 4, 1], V, seed=V, sigma=2.0)
@@ -163,7 +163,8 @@ def test_blank_positions(blank, fused):
 
 @pytest.mark.parametrize("dtype,V", [("f16", 64), ("f16", 4096), ("bf16", 256), ("f64", 32), ("f64", 1024),
                                      ("f16", 5537), ("f16", 520), ("bf16", 4233), ("f64", 777), ("f16", 32000),
-                                     ("f16", 41), ("bf16", 100), ("f64", 33), ("f16", 7)])
+                                     ("f16", 41), ("bf16", 100), ("f64", 33), ("f16", 7), ("f16", 512), ("bf16", 1024),
+                                     ("f16", 200), ("f64", 100), ("f64", 256)])
 @pytest.mark.parametrize("fused", [False, True])
 def test_storage_types(dtype, V, fused):
     b = make_batch([12, 5, 20], [4, 7, 2], V, seed=V, dtype=dtype, normalised=not fused)
