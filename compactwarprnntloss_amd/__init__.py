@@ -5,7 +5,8 @@ the work is done by hand-written HIP kernels behind the C ABI of include/cwarp_r
 """
 from .loss import (ForwardState, lattice_state, pack_padded, rnnt_backward, rnnt_forward,  # noqa: F401
                    rnnt_loss, transducer_loss)
+from .joiner import CompactJoiner, compact_join  # noqa: F401
 
 __version__ = "0.1.0"
 __all__ = ["transducer_loss", "rnnt_loss", "pack_padded", "lattice_state", "rnnt_forward", "rnnt_backward",
-           "ForwardState", "__version__"]
+           "ForwardState", "compact_join", "CompactJoiner", "__version__"]

@@ -350,4 +350,41 @@ int cwr_unpack(const void* g_compact, int dtype, int64_t N, int64_t T_pad, int64
     return repack_impl(g_compact, g_padded, dtype, N, T_pad, Up_pad, V, lx, ly, row_off, R, nullptr, stream, true);
 }
 
+static int join_check(int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t H, int64_t R,
+                      const int32_t* lx, const int32_t* ly, const int64_t* row_off) {
+    if (dtype < CWR_F32 || dtype > CWR_F64) return CWR_ERR_DTYPE;
+    if (act < CWR_ACT_NONE || act > CWR_ACT_RELU) return CWR_ERR_MODE;
+    if (N < 0 || T_pad < 0 || Up_pad < 0 || H < 1 || R < 0) return CWR_ERR_SHAPE;
+    if (N > 0x3fffffff || H > 0x3fffffff || T_pad > 0x3fffffff || Up_pad > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (N > 0 && (!lx || !ly || !row_off)) return CWR_ERR_NULL;
+    if (misaligned(lx, 4) || misaligned(ly, 4) || misaligned(row_off, 8)) return CWR_ERR_ALIGN;
+    return CWR_OK;
+}
+
+int cwr_join(const void* f, const void* g, int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t H,
+             const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* h, int32_t* status,
+             void* stream) {
+    int rc = join_check(dtype, act, N, T_pad, Up_pad, H, R, lx, ly, row_off);
+    if (rc != CWR_OK) return rc;
+    if (N > 0 && T_pad > 0 && Up_pad > 0 && (!f || !g)) return CWR_ERR_NULL;
+    if (R > 0 && !h) return CWR_ERR_NULL;
+    const size_t es = elem_size(dtype);
+    if (misaligned(f, es) || misaligned(g, es) || misaligned(h, es) || misaligned(status, 4)) return CWR_ERR_ALIGN;
+    return launch_join(dtype, act, false, f, g, h, nullptr, lx, ly, reinterpret_cast<const i64*>(row_off), N, T_pad,
+                       Up_pad, H, R, status, static_cast<hipStream_t>(stream));
+}
+
+int cwr_join_backward(const void* dh, const void* h, int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad,
+                      int64_t H, const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* df,
+                      void* dg, void* stream) {
+    int rc = join_check(dtype, act, N, T_pad, Up_pad, H, R, lx, ly, row_off);
+    if (rc != CWR_OK) return rc;
+    if (R > 0 && (!dh || (act != CWR_ACT_NONE && !h))) return CWR_ERR_NULL;
+    if (N > 0 && ((T_pad > 0 && !df) || (Up_pad > 0 && !dg))) return CWR_ERR_NULL;
+    const size_t es = elem_size(dtype);
+    if (misaligned(dh, es) || misaligned(h, es) || misaligned(df, es) || misaligned(dg, es)) return CWR_ERR_ALIGN;
+    return launch_join(dtype, act, true, dh, h, df, dg, lx, ly, reinterpret_cast<const i64*>(row_off), N, T_pad,
+                       Up_pad, H, R, nullptr, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -81,6 +81,12 @@ int launch_export(const int* lx, const int* ly, int N, i64 T_pad, i64 Up_pad, co
 int launch_repack(const void* src, void* dst, size_t esize, const int* lx, const int* ly, const i64* row_off, i64 N,
                   i64 T_pad, i64 Up_pad, i64 V, i64 R, bool unpack, int* status, hipStream_t stream);
 
+// forward (backward = false): a = f, b = g, o1 = out; backward: a = dh, b = h (unused without an
+// activation), o1 = df, o2 = dg
+int launch_join(int dtype, int act, bool backward, const void* a, const void* b, void* o1, void* o2, const int* lx,
+                const int* ly, const i64* row_off, i64 N, i64 T_pad, i64 Up_pad, i64 H, i64 R, int* status,
+                hipStream_t stream);
+
 inline int check_launch() {
     return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;
 }

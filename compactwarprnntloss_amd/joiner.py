@@ -1,0 +1,96 @@
+"""Compact joiner: the step that produces the (sum_i T_i*(U_i+1), V) rows the loss consumes.
+
+The reference repository holds no joiner; its callers form the padded (N, T, U+1, H) broadcast sum
+of encoder frames and predictor states, run the output layer over all of it and pass padded logits
+to cwarp_rnnt/__init__.py:52-59.  `compact_join` forms the sum for the cells of each sequence's own
+lattice only, directly in the compact row order of test/test.py:44-46 (kernels in csrc/join.hip,
+entry points cwr_join / cwr_join_backward); the output layer is then a plain GEMM over (R, H) rows,
+which `CompactJoiner` leaves to torch (hipBLASLt)."""
+from typing import Any, Optional
+
+import torch
+
+from . import _lib
+from .loss import _DTYPES, _offsets, _stream_ptr
+
+_ACTS = {None: 0, "none": 0, "tanh": 1, "relu": 2}
+
+
+class _Join(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx: Any, f, g, lx, ly, total_rows, act):
+        lib = _lib.load()
+        N, T, H = f.shape
+        Up = g.size(1)
+        row_off, status = _offsets(lx, ly, total_rows)
+        out = torch.empty((total_rows, H), dtype=f.dtype, device=f.device)
+        with torch.cuda.device(f.device):
+            rc = lib.cwr_join(f.data_ptr(), g.data_ptr(), _DTYPES[f.dtype], act, N, T, Up, H, lx.data_ptr(),
+                              ly.data_ptr(), row_off.data_ptr(), total_rows, out.data_ptr(), status.data_ptr(),
+                              _stream_ptr(f.device))
+            _lib.check(rc, "cwr_join")
+        ctx.save_for_backward(lx, ly, row_off, out if act else None)
+        ctx.dims = (N, T, Up, H)
+        ctx.act = act
+        ctx.status = status
+        return out
+
+    @staticmethod
+    def backward(ctx: Any, dh):
+        lx, ly, row_off, out = ctx.saved_tensors
+        N, T, Up, H = ctx.dims
+        lib = _lib.load()
+        dh = dh.contiguous()
+        df = torch.empty((N, T, H), dtype=dh.dtype, device=dh.device)
+        dg = torch.empty((N, Up, H), dtype=dh.dtype, device=dh.device)
+        with torch.cuda.device(dh.device):
+            rc = lib.cwr_join_backward(dh.data_ptr(), out.data_ptr() if out is not None else None,
+                                       _DTYPES[dh.dtype], ctx.act, N, T, Up, H, lx.data_ptr(), ly.data_ptr(),
+                                       row_off.data_ptr(), dh.size(0), df.data_ptr(), dg.data_ptr(),
+                                       _stream_ptr(dh.device))
+            _lib.check(rc, "cwr_join_backward")
+        return df, dg, None, None, None, None
+
+
+def compact_join(f: torch.Tensor, g: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
+                 activation: Optional[str] = None, total_rows: Optional[int] = None) -> torch.Tensor:
+    """h[row(n,t,u), :] = act(f[n, t, :] + g[n, u, :]) for t < lx[n], u <= ly[n], as (R, H) compact
+    rows (sequence-major, then t, then u).  Differentiable in f and g.
+
+    f: (N, T, H) encoder frames; g: (N, U+1, H) predictor states; lx, ly: (N,) int32 frame and label
+    counts; activation: None, "tanh" or "relu"; total_rows: sum_i lx_i*(ly_i+1) if known, else it is
+    computed on the device and read back (one synchronisation)."""
+    if activation not in _ACTS:
+        raise RuntimeError(f"activation must be one of {sorted(k for k in _ACTS if k)} or None")
+    if f.dim() != 3 or g.dim() != 3 or f.size(0) != g.size(0) or f.size(2) != g.size(2):
+        raise RuntimeError("f must be (N, T, H) and g (N, U+1, H)")
+    if f.dtype != g.dtype or f.dtype not in _DTYPES:
+        raise RuntimeError(f"f and g must share a supported dtype, got {f.dtype} and {g.dtype}")
+    if not f.is_cuda or not g.is_cuda:
+        raise RuntimeError("f and g must be CUDA tensors")
+    for name, t in (("lx", lx), ("ly", ly)):
+        if not t.is_cuda or t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous CUDA int32 tensor")
+    if lx.numel() != f.size(0) or ly.numel() != f.size(0):
+        raise RuntimeError("lx, ly must hold one entry per sequence")
+    if total_rows is None:
+        total_rows = int((lx.long() * (ly.long() + 1)).sum().item())
+    return _Join.apply(f.contiguous(), g.contiguous(), lx, ly, int(total_rows), _ACTS[activation])
+
+
+class CompactJoiner(torch.nn.Module):
+    """Projection of encoder and predictor outputs to a joint space, their compact broadcast sum
+    with an activation, and the output layer: (N,T,E), (N,U+1,P) -> (R, V) logits in the layout
+    `transducer_loss(..., fused_log_softmax=True)` takes.  The three linear layers are library
+    GEMMs; only the sum is done here, and only for the cells the loss will read."""
+
+    def __init__(self, enc_dim: int, pred_dim: int, joint_dim: int, vocab: int, activation: str = "tanh"):
+        super().__init__()
+        self.enc = torch.nn.Linear(enc_dim, joint_dim)
+        self.pred = torch.nn.Linear(pred_dim, joint_dim, bias=False)
+        self.out = torch.nn.Linear(joint_dim, vocab)
+        self.activation = activation
+
+    def forward(self, enc_out, pred_out, lx, ly, total_rows: Optional[int] = None):
+        h = compact_join(self.enc(enc_out), self.pred(pred_out), lx, ly, self.activation, total_rows)
+        return self.out(h)

@@ -211,6 +211,27 @@ int cwr_unpack(const void* g_compact, int dtype, int64_t N, int64_t T_pad, int64
                const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* g_padded,
                void* stream);
 
+/* Compact joiner front: h[row_off[n] + t*(ly[n]+1) + u, :] = act(f[n, t, :] + g[n, u, :]) for
+ * t < lx[n], u <= ly[n] -- the broadcast sum of encoder frames and predictor states for the cells
+ * of each sequence's own lattice only, in the compact row order of test/test.py:44-46.  The
+ * reference repository has no joiner (its callers form the padded (N,T,U+1,H) sum and pass padded
+ * logits to cwarp_rnnt/__init__.py:52-59); the linear layer that follows is left to a library GEMM
+ * over the (R, H) rows.
+ *   f (N, T_pad, H), g (N, Up_pad, H) contiguous;  h (R, H);  act a cwr_activation
+ *   status as for cwr_pack. */
+enum cwr_activation { CWR_ACT_NONE = 0, CWR_ACT_TANH = 1, CWR_ACT_RELU = 2 };
+int cwr_join(const void* f, const void* g, int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t H,
+             const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* h, int32_t* status,
+             void* stream);
+
+/* Backward of cwr_join: df[n, t, :] = sum over u of dz, dg[n, u, :] = sum over t of dz, where
+ * dz = dh * act'(z) with act' taken from the stored output h (unused, may be NULL, for
+ * CWR_ACT_NONE).  Sums run in a fixed order (no atomics); every element of df and dg is written,
+ * zeros outside each sequence's lattice. */
+int cwr_join_backward(const void* dh, const void* h, int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad,
+                      int64_t H, const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* df,
+                      void* dg, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

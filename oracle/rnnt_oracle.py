@@ -32,6 +32,9 @@ tests/test_oracle_pins.py:
                                 torch.autograd through an independent torch restatement
   dense gradients (both modes)  finite differences of the full function; rows sum to zero (fused
                                 mode); linearity in grad_out
+  join_rows / join_rows_backward  (no reference counterpart: the repository has no joiner)
+                                padded broadcast sum packed by compact_from_padded; central finite
+                                differences
 
 Two gradient definitions are provided:
   mode "logprob"  x already holds log-probabilities (what the reference computes): the gradient
@@ -83,6 +86,58 @@ def compact_from_padded(xp, lx, ly):
     for n in range(xp.shape[0]):
         out.append(xp[n, : lx[n], : ly[n] + 1, :].reshape(-1, xp.shape[-1]))
     return np.concatenate(out, axis=0)
+
+
+def _activation(z, act):
+    if act in (None, "none"):
+        return z
+    if act == "tanh":
+        return np.tanh(z)
+    if act == "relu":
+        return np.maximum(z, 0.0)
+    raise ValueError(act)
+
+
+def join_rows(f, g, lx, ly, act=None):
+    """Compact joiner front: one (H,) row act(f[n,t] + g[n,u]) per lattice cell, in the compact row
+    order (test/test.py:44-46).  The reference repository has no joiner; this restates what its
+    callers feed cwarp_rnnt/__init__.py:52-59 (a padded broadcast sum), restricted to valid cells.
+    f: (N,Tmax,H), g: (N,Umax+1,H).  Written cell by cell; pinned against the padded broadcast sum
+    packed by compact_from_padded."""
+    f = np.asarray(f, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    rows = []
+    for n in range(f.shape[0]):
+        for t in range(int(lx[n])):
+            for u in range(int(ly[n]) + 1):
+                rows.append(_activation(f[n, t] + g[n, u], act))
+    if not rows:
+        return np.zeros((0, f.shape[-1]))
+    return np.stack(rows)
+
+
+def join_rows_backward(dh, f, g, lx, ly, act=None):
+    """Gradient of sum(dh * join_rows(f, g)) w.r.t. f and g: dz = dh * act'(z) summed over u for f
+    and over t for g, zeros in the padding.  Pinned by central finite differences."""
+    f = np.asarray(f, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    dh = np.asarray(dh, dtype=np.float64)
+    df, dg = np.zeros_like(f), np.zeros_like(g)
+    r = 0
+    for n in range(f.shape[0]):
+        for t in range(int(lx[n])):
+            for u in range(int(ly[n]) + 1):
+                z = f[n, t] + g[n, u]
+                if act == "tanh":
+                    dz = dh[r] * (1.0 - np.tanh(z) ** 2)
+                elif act == "relu":
+                    dz = dh[r] * (z > 0)
+                else:
+                    dz = dh[r]
+                df[n, t] += dz
+                dg[n, u] += dz
+                r += 1
+    return df, dg
 
 
 def labels_of(y, ly, n):

@@ -137,6 +137,19 @@ def test_invalid_calls_are_rejected_on_the_host():
     assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, None, 1 << 30, 4, 4, p(3), p(4), None) == 1
     assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, p(5), 16, 4, 4, p(3), p(4), None) == 4  # workspace too small
     assert lib.cwr_export_lattice(p(1), p(2), 2, 10, 3, p(5), 1 << 30, 4, 4, None, None, None) == 1
+    # cwr_join(f, g, dtype, act, N, T_pad, Up_pad, H, lx, ly, row_off, R, h, status, stream)
+    assert lib.cwr_join(None, p(2), 0, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), None, None) == 1
+    assert lib.cwr_join(p(1), p(2), 0, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, None, None, None) == 1
+    assert lib.cwr_join(p(1), p(2), 5, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), None, None) == 2
+    assert lib.cwr_join(p(1), p(2), 0, 3, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), None, None) == 3   # activation
+    assert lib.cwr_join(p(1), p(2), 0, 0, 2, 3, 4, 0, p(3), p(4), p(5), 10, p(6), None, None) == 4
+    assert lib.cwr_join(p(1), p(2), 0, 0, 2, 3, 4, 8, None, p(4), p(5), 10, p(6), None, None) == 1
+    assert lib.cwr_join(p(1) + 2, p(2), 0, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), None, None) == 6
+    assert lib.cwr_join_backward(None, None, 0, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), p(7), None) == 1
+    assert lib.cwr_join_backward(p(1), None, 0, 1, 2, 3, 4, 8, p(3), p(4), p(5), 10, p(6), p(7), None) == 1  # tanh needs h
+    assert lib.cwr_join_backward(p(1), None, 0, 0, 2, 3, 4, 8, p(3), p(4), p(5), 10, None, p(7), None) == 1
+    assert lib.cwr_join_backward(p(1), p(2), 0, 2, 2, 1 << 31, 4, 8, p(3), p(4), p(5), 10, p(6), p(7), None) == 8
+    assert lib.cwr_join(None, None, 0, 0, 0, 0, 0, 8, None, None, None, 0, None, None, None) == 0   # empty batch
     # R == 0 is a valid (empty) call and launches nothing that touches memory
     assert lib.cwr_backward(None, 0, 0, 8, None, None, None, 0, 0, 0, 0, 0, None, None, None, None, None,
                             None, 1, 1.0, None, None) == 0

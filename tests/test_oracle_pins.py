@@ -299,3 +299,37 @@ def test_configs_are_seeded_and_in_range():
     assert c4["ly"].min() == 0 and c4["lx"].min() == 1 and c4["N"] == 64
     c2 = orc.make_config(2)
     assert c2["N"] == 32 and c2["V"] == 1024 and 100 <= c2["lx"].min() and c2["lx"].max() <= 250
+
+
+# ----------------------------------------------------------------------------- joiner front
+@pytest.mark.parametrize("act", [None, "tanh", "relu"])
+def test_join_rows_equal_packed_broadcast_sum(act):
+    rng = np.random.default_rng(11)
+    lx, ly = np.array([3, 1, 5]), np.array([2, 0, 4])
+    f = rng.normal(size=(3, 5, 6))
+    g = rng.normal(size=(3, 5, 6))
+    z = f[:, :, None, :] + g[:, None, :, :]
+    full = {None: z, "tanh": np.tanh(z), "relu": np.maximum(z, 0)}[act]
+    np.testing.assert_array_equal(orc.join_rows(f, g, lx, ly, act), orc.compact_from_padded(full, lx, ly))
+
+
+@pytest.mark.parametrize("act", [None, "tanh", "relu"])
+def test_join_rows_backward_matches_finite_differences(act):
+    rng = np.random.default_rng(12)
+    lx, ly = np.array([2, 3]), np.array([1, 2])
+    f = rng.normal(size=(2, 4, 3))   # one padded frame / state in each array
+    g = rng.normal(size=(2, 4, 3))
+    R = int((lx * (ly + 1)).sum())
+    dh = rng.normal(size=(R, 3))
+    df, dg = orc.join_rows_backward(dh, f, g, lx, ly, act)
+    fn = lambda a, b: float((dh * orc.join_rows(a, b, lx, ly, act)).sum())
+    eps = 1e-6
+    for arr, grad, which in ((f, df, 0), (g, dg, 1)):
+        num = np.zeros_like(arr)
+        for idx in np.ndindex(arr.shape):
+            p, m = arr.copy(), arr.copy()
+            p[idx] += eps
+            m[idx] -= eps
+            num[idx] = ((fn(p, g) - fn(m, g)) if which == 0 else (fn(f, p) - fn(f, m))) / (2 * eps)
+        np.testing.assert_allclose(grad, num, atol=1e-7)
+    assert np.all(df[0, 2:] == 0) and np.all(dg[0, 2:] == 0)   # padding gets no gradient
