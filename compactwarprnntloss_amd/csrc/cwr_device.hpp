@@ -151,11 +151,9 @@ template <> struct Elem<bf16_t> {
     static constexpr int VEC = 8;
     static __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.v << 16); }
     static __device__ __forceinline__ bf16_t from_f32(float f) {
-        uint32_t u = __float_as_uint(f);
+        const __bf16 h = (__bf16)f;  // gfx950's conversion instruction: round to nearest even, NaN kept
         bf16_t r;
-        if ((u & 0x7fffffffu) > 0x7f800000u) { r.v = (uint16_t)((u >> 16) | 0x40); return r; }  // NaN
-        u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-        r.v = (uint16_t)(u >> 16);
+        __builtin_memcpy(&r.v, &h, 2);
         return r;
     }
 };

@@ -27,16 +27,6 @@ template <typename T> struct Arith {
     static __device__ __forceinline__ float up(T v) { return Elem<T>::to_f32(v); }
     static __device__ __forceinline__ T down(float v) { return Elem<T>::from_f32(v); }
 };
-template <> struct Arith<bf16_t> {
-    typedef float type;
-    static __device__ __forceinline__ float up(bf16_t v) { return Elem<bf16_t>::to_f32(v); }
-    static __device__ __forceinline__ bf16_t down(float v) {  // the conversion instruction (round to nearest even)
-        const __bf16 h = (__bf16)v;
-        bf16_t r;
-        __builtin_memcpy(&r, &h, 2);
-        return r;
-    }
-};
 template <> struct Arith<double> {
     typedef double type;
     static __device__ __forceinline__ double up(double v) { return v; }
