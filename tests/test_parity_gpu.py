@@ -408,6 +408,40 @@ def test_more_than_64_sequences(fused, V):
     check_case(b, fused, "1d")
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_rows_beyond_two_to_the_31_elements(fused):
+    """A tensor of more than 2^31 elements (the reference's int32 offsets end there,
+    cwarp_cuda.cpp:72-77): the sequences at its far end must give the same costs and gradient
+    rows as when they are run as a small batch of their own, and so must the first ones."""
+    pkg = _pkg()
+    N, T, U, V = 32, 700, 99, 1024
+    R = N * T * (U + 1)
+    assert R * V > 2 ** 31
+    DEV = torch.device("cuda:0")
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    x = torch.randn((R, V), device=DEV, dtype=torch.float16, generator=gen)
+    if not fused:
+        x = x.sub_(torch.logsumexp(x[:4096].float(), dim=1).mean().half())  # roughly normalised is enough here
+    y = torch.randint(1, V, (N, U), device=DEV, dtype=torch.int32, generator=gen)
+    lx = torch.full((N,), T, dtype=torch.int32, device=DEV)
+    ly = torch.full((N,), U, dtype=torch.int32, device=DEV)
+    costs, st = pkg.rnnt_forward(x, lx, y, ly, 0, fused)
+    go = torch.ones(N, device=DEV)
+    g = pkg.rnnt_backward(x, lx, y, ly, 0, st, go)
+    assert int(st.status[0].item()) & ~8 == 0
+    rows = T * (U + 1)
+    for sl in (slice(0, 2), slice(N - 2, N)):
+        xs = x[sl.start * rows: sl.stop * rows]
+        c2, st2 = pkg.rnnt_forward(xs, lx[sl].contiguous(), y[sl].contiguous(), ly[sl].contiguous(), 0, fused)
+        g2 = pkg.rnnt_backward(xs, lx[sl].contiguous(), y[sl].contiguous(), ly[sl].contiguous(), 0, st2, go[sl].contiguous())
+        torch.testing.assert_close(costs[sl], c2, rtol=1e-6, atol=0)
+        assert torch.equal(g[sl.start * rows: sl.stop * rows], g2)
+    assert torch.isfinite(costs).all()
+    if fused:   # rows of the dense gradient sum to zero, also at the far end
+        tail = g[-4096:].float().sum(dim=1)
+        assert float(tail.abs().max()) < 2e-2   # 1024 fp16-rounded entries per row
+
+
 # ----------------------------------------------------------------------------- number systems of the lattice walk
 def _walk_modes(st):
     """Per-sequence walk-mode words of a forward call (workspace section 4)."""
