@@ -133,7 +133,7 @@ using namespace cwr;
 
 extern "C" {
 
-int cwr_version(void) { return 120; }
+int cwr_version(void) { return 130; }
 
 const char* cwr_strerror(int status) {
     switch (status) {

@@ -149,3 +149,26 @@ def test_join_rejects_bad_arguments():
         pkg.compact_join(f, g.half(), l, l)
     with pytest.raises(RuntimeError):
         pkg.compact_join(f, g, l.long(), l)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_join_and_pack_random_batches(seed):
+    """Random batch shapes (1 to 100 sequences, empty label sequences, rows on and off the 16-byte
+    grid, padded widths wider than needed): compact_join against the oracle, and pack_padded of the
+    padded broadcast sum bit-exact against compact_join."""
+    pkg = _pkg()
+    rng = np.random.default_rng(100 + seed)
+    N = int(rng.integers(1, 101))
+    lx = rng.integers(1, 14, N).astype(np.int32)
+    ly = rng.integers(0, 9, N).astype(np.int32)
+    H = int(rng.choice([4, 7, 24, 64, 100, 256, 260]))
+    dtype = str(rng.choice(["f32", "f16", "bf16", "f64"]))
+    lx_, ly_, f, g = _inputs(lx, ly, H, dtype, seed=seed, t_extra=int(rng.integers(0, 3)), u_extra=int(rng.integers(0, 3)))
+    fd, gd = f.to(DEV), g.to(DEV)
+    lxd, lyd = torch.from_numpy(lx).to(DEV), torch.from_numpy(ly).to(DEV)
+    h = pkg.compact_join(fd, gd, lxd, lyd, None)
+    ref = orc.join_rows(f.double().numpy(), g.double().numpy(), lx, ly, None)
+    np.testing.assert_allclose(h.double().cpu().numpy(), ref, rtol=ROUND[dtype] * 2, atol=ROUND[dtype] * 4)
+    acc = torch.float64 if dtype == "f64" else torch.float32
+    z = (fd.to(acc)[:, :, None, :] + gd.to(acc)[:, None, :, :]).to(fd.dtype).contiguous()
+    assert torch.equal(pkg.pack_padded(z, lxd, lyd), h)
