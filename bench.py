@@ -93,6 +93,10 @@ def main():
     ap.add_argument("--with-pack", action="store_true",
                     help="also time the padded -> compact pack op and its backward on the padded form of the same "
                          "batch (reported under 'pack_op'; not part of 'value')")
+    ap.add_argument("--with-joiner", action="store_true",
+                    help="also time the compact joiner front (broadcast sum + tanh for valid cells, H=512, in the "
+                         "batch's storage type) and its backward at the same lengths (reported under 'joiner_op'; "
+                         "not part of 'value')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so that a counter run can scale "
                          "FETCH_SIZE / WRITE_SIZE against it")
@@ -212,6 +216,33 @@ def main():
             "pack_GBs": round(2 * R * V * esize / (pack_ms * 1e-3) / 1e9, 1),
             "unpack_GBs": round((R * V * esize + padded_bytes) / (unpack_ms * 1e-3) / 1e9, 1)}
         del x4, g4, packed
+
+    if args.with_joiner:
+        H = 512
+        lib = pkg._lib.load()
+        Tm, Up = int(cfg["lx"].max()), int(cfg["ly"].max()) + 1
+        f = torch.randn((N, Tm, H), device=dev).to(tdt)
+        g = torch.randn((N, Up, H), device=dev).to(tdt)
+        row_off, _st = pkg.loss._offsets(lx, ly, R)
+        h = torch.empty((R, H), dtype=tdt, device=dev)
+        dh = torch.randn((R, H), device=dev).to(tdt)
+        df, dg = torch.empty_like(f), torch.empty_like(g)
+        dt = pkg.loss._DTYPES[tdt]
+        stream = torch.cuda.current_stream().cuda_stream
+        ops = {}
+        for name, act in (("sum", 0), ("tanh", 1)):
+            fw = timed(lambda: lib.cwr_join(f.data_ptr(), g.data_ptr(), dt, act, N, Tm, Up, H, lx.data_ptr(),
+                                            ly.data_ptr(), row_off.data_ptr(), R, h.data_ptr(), None, stream))
+            bw = timed(lambda: lib.cwr_join_backward(dh.data_ptr(), h.data_ptr(), dt, act, N, Tm, Up, H,
+                                                     lx.data_ptr(), ly.data_ptr(), row_off.data_ptr(), R,
+                                                     df.data_ptr(), dg.data_ptr(), stream))
+            rb = R * H * esize
+            # forward: the (R,H) rows stored; backward: dh (and h with an activation) read once per sum
+            ops[name] = {"forward_ms": round(fw, 4), "backward_ms": round(bw, 4),
+                         "forward_GBs": round(rb / (fw * 1e-3) / 1e9, 1),
+                         "backward_GBs": round((2 if act == 0 else 4) * rb / (bw * 1e-3) / 1e9, 1)}
+        result["joiner_op"] = {"H": H, "rows": R, **ops}
+        del f, g, h, dh, df, dg
 
     if not args.no_cpu:
         g_all = pkg.rnnt_backward(xd, lx, y, ly, 0, st, go, out=out)
