@@ -817,13 +817,22 @@ __device__ __forceinline__ bool fill_slot(const int* __restrict__ lx, const int*
         }
         if (slot >= total) return false;
     } else {
-        if (slot >= slot_off[N]) return false;
+        // the wave's first slot is placed by a search on the scalar unit; its lanes step on from
+        // there over the few boundaries inside the wave's 64 slots (wave-uniform loads)
+        const i64 s0 = (i64)blockIdx.x * 256 + (__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) << 6);
+        if (s0 >= slot_off[N]) return false;
         int lo = 0, hi = N;
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
-            if (slot_off[mid] <= slot) lo = mid; else hi = mid;
+            if (slot_off[mid] <= s0) lo = mid; else hi = mid;
         }
         n = lo;
+        for (int j = lo + 1; j < N; ++j) {
+            const i64 oj = slot_off[j];
+            if (oj > s0 + 63) break;
+            n += oj <= slot ? 1 : 0;
+        }
+        if (slot >= slot_off[N]) return false;
     }
     const i64 pad = pad_off[n];
     if (pad < 0) return false;

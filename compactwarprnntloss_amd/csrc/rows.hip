@@ -375,9 +375,25 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
                 ri.u = (int)(rem - (i64)ri.t * (U_ + 1));
             }
         }
-    } else if (mine) {
-        ri = decode_row(r, R, row_off, lx, ly, N);
-        if (ri.n >= 0) { pad = pad_off[ri.n]; labbase = lab_off[ri.n]; }
+    } else {
+        // more sequences than lanes: the wave's first row is placed by a search on the scalar unit
+        // and the lanes step on from there (the offsets they step over are wave-uniform loads)
+        int lo = 0, hi = N - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (row_off[mid] <= r0) lo = mid; else hi = mid - 1;
+        }
+        int n = lo;
+        const i64 r_last = r0 + ROWS - 1;
+        for (int j = lo + 1; j < N; ++j) {
+            const i64 oj = row_off[j];
+            if (oj > r_last) break;
+            n += (mine && oj <= r) ? 1 : 0;
+        }
+        if (mine) {
+            ri = place_row(r, n, R, row_off, lx, ly);
+            if (ri.n >= 0) { pad = pad_off[n]; labbase = lab_off[n]; }
+        }
     }
     int my_lab = -1;
     i64 my_dst = -1;

@@ -396,7 +396,7 @@ def test_full_size_configs_against_oracle(idx):
     assert float(np.abs(g.cpu().numpy() - ref["grad"]).max()) <= GRAD_ATOL
 
 
-@pytest.mark.parametrize("fused,V", [(True, 64), (True, 1024), (False, 40)])
+@pytest.mark.parametrize("fused,V", [(True, 64), (True, 128), (True, 512), (True, 1024), (False, 40)])
 def test_more_than_64_sequences(fused, V):
     """Batches beyond 64 sequences leave the in-register sequence tables (gather, fill) for the
     search over the offset arrays."""
