@@ -117,13 +117,36 @@ template <> struct Pack<double> {
 // two as plain probabilities for the scaled linear-domain walk.  A logarithm outside
 // [kLinMin, kLinMax] cannot be carried by that walk within one of its blocks (nor, as a
 // probability, by fp32); the sequence is then marked for the log-domain walk.
-__device__ __forceinline__ LpCell make_lp(float xb, float xl, float lse, bool has_label, int* seqmode_n) {
-    const float b = (float)(((double)fmaxf(xb, kLpFloor) - (double)lse) * 1.4426950408889634);
-    const float l = has_label ? (float)(((double)fmaxf(xl, kLpFloor) - (double)lse) * 1.4426950408889634) : 0.f;
+// A row's log-sum-exp as (maximum m, log2 of the sum of exp(x - m)).  Kept in two parts for the
+// cell records: x - m is exact and log2(sum) is small when a row is peaked, so that a
+// log-probability close to zero keeps its absolute accuracy however large the logits are (one
+// fp32 number m + ln(sum) would carry half an ulp of m into every log-probability).
+struct Lse {
+    float m, l2s;
+    __device__ __forceinline__ float value() const { return fmaf(l2s, kLn2, m); }
+};
+// log2 of a sum s >= 1 of exponentials whose largest term is 1, and 2^b for a log-probability b:
+// series next to s = 1 and b = 0, where the hardware approximations are good to an ulp of their
+// RESULT's neighbourhood (about 1e-7 absolute) but a peaked row needs the small difference itself.
+__device__ __forceinline__ float log2_of_sum(float s) {
+    const float d = s - 1.f;  // exact for s in [1, 2]
+    const float series = d * fmaf(d, fmaf(d, 1.f / 3.f, -0.5f), 1.f) * kLog2e;
+    return d < 0.015625f ? series : fast_log2(s);
+}
+__device__ __forceinline__ float exp2_of_logprob(float b) {
+    const float z = b * kLn2;
+    const float series = fmaf(z, fmaf(z, fmaf(z, 1.f / 6.f, 0.5f), 1.f), 1.f);
+    return b > -0.015625f ? series : fast_exp2(b);
+}
+
+__device__ __forceinline__ LpCell make_lp(float xb, float xl, const Lse lse, bool has_label, int* seqmode_n) {
+    const float b = (float)(((double)fmaxf(xb, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s);
+    const float l = has_label
+        ? (float)(((double)fmaxf(xl, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s) : 0.f;
     if (!(b >= kLinMin && b <= kLinMax && l >= kLinMin && l <= kLinMax)) atomicOr(seqmode_n, 1);
     LpCell c;
-    c.p_blank = fast_exp2(b);
-    c.p_label = fast_exp2(l);
+    c.p_blank = exp2_of_logprob(b);
+    c.p_label = exp2_of_logprob(l);
     c.l_blank = b;
     c.l_label = l;
     return c;
@@ -161,7 +184,7 @@ template <int LPR> __device__ __forceinline__ float lane_get(float v, int i) {
 // row's log-sum-exp and its blank / label entries.
 template <typename T, int LPR, int K, bool EXTRACT = true>
 __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, const ColPos<Elem<T>::VEC, LPR>& pb,
-                                            const int lab, float& lse, float& xb, float& xl) {
+                                            const int lab, Lse& lse, float& xb, float& xl) {
     constexpr int VEC = Elem<T>::VEC;
     typename RegVec<K * VEC>::type xv;
 #pragma unroll
@@ -181,7 +204,10 @@ __device__ __forceinline__ void gather_pass(const v4i (&raw)[K], const int g, co
 #pragma unroll
         for (int j = 0; j < K * VEC; ++j) s += fast_exp2(fmaf(xv[j], kLog2e, -ms));
         s = group_allreduce<LPR, OpSum>(s);
-        lse = fmaf(fast_log2(s), kLn2, m);
+        lse.m = m;
+        // every exponent above is off by what ms lost to rounding (up to half an ulp of m log2 e,
+        // 2e-6 for m = 25): the fma below recovers it exactly
+        lse.l2s = log2_of_sum(s) - fmaf(m, kLog2e, -ms);
     }
     if (!EXTRACT) return;
     // pick the blank and label entries out of the registers
@@ -282,11 +308,12 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     for (int k = 0; k < K; ++k)
         if (lane + k * 64 >= NV) raw[k] = Pack<T>::neg_inf();
     const ColPos<VEC, 64> pb(blank);
-    float lse, rb, rl;
+    Lse lse;
+    float rb, rl;
     gather_pass<T, 64, K, kFromRegs>(raw, 0, pb, lab, lse, rb, rl);
     if (kFromRegs) { xb = rb; xl = rl; }
     if (lane == 0) {
-        lse_out[r] = lse;
+        lse_out[r] = lse.value();
         rowinfo[r] = make_int2(lab, ri.n);
         if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
@@ -407,7 +434,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     }
 
     const ColPos<VEC, LPR> pb(blank);
-    float res_lse = 0.f, res_b = 0.f, res_l = 0.f;  // results of the lane's own row
+    Lse res_lse = {0.f, 0.f};
+    float res_b = 0.f, res_l = 0.f;  // results of the lane's own row
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const bool ok = r0 + p * RP + g < R;
@@ -422,15 +450,17 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         } else {
             lab = __shfl(my_lab, g * LPR + p);
         }
-        float lse, xb, xl;
+        Lse lse;
+        float xb, xl;
         gather_pass<T, LPR, K>(raw[p], g, pb, lab, lse, xb, xl);
         const bool here = lir == p;
-        res_lse = here ? lse : res_lse;
+        res_lse.m = here ? lse.m : res_lse.m;
+        res_lse.l2s = here ? lse.l2s : res_lse.l2s;
         res_b = here ? xb : res_b;
         res_l = here ? xl : res_l;
     }
     if (mine) {
-        lse_out[r] = res_lse;
+        lse_out[r] = res_lse.value();
         rowinfo[r] = make_int2(my_lab, ri.n);
         if (my_dst >= 0) lp[my_dst] = make_lp(res_b, res_l, res_lse, my_lab >= 0, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
@@ -510,10 +540,14 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
         }
         if (m > -INFINITY) {
             const float ms = m * kLog2e;
+            float cs = 0.f;
 #pragma unroll
             for (int k = 0; k < KC; ++k)
 #pragma unroll
-                for (int c = 0; c < VEC; ++c) s += fast_exp2(fmaf(xv[k][c], kLog2e, -ms));
+                for (int c = 0; c < VEC; ++c) cs += fast_exp2(fmaf(xv[k][c], kLog2e, -ms));
+            // the exponents are off by what ms lost to rounding, the same for the whole chunk: the
+            // fma recovers it exactly and the chunk's sum is brought back to the scale of m
+            s = fmaf(cs, fmaf(-fmaf(m, kLog2e, -ms), kLn2, 1.f), s);
         }
     };
     // two buffers taking turns, so that no register with a load in flight is ever copied
@@ -536,9 +570,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
     }
     const float M = group_allreduce<64, OpMax>(m);
     const float S = group_allreduce<64, OpSum>(m > -INFINITY ? s * fast_exp2((m - M) * kLog2e) : 0.f);
-    const float lse = fmaf(fast_log2(S), kLn2, M);
+    const Lse lse = {M, log2_of_sum(S)};
     if (lane == 0) {
-        lse_out[r] = lse;
+        lse_out[r] = lse.value();
         rowinfo[r] = make_int2(lab, ri.n);
         if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
@@ -576,9 +610,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_small(
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) s += fast_exp2(fmaf(xv[k], kLog2e, -ms));
     s = group_allreduce<LPR, OpSum>(s);
-    const float lse = fmaf(fast_log2(s), kLn2, m);
+    const Lse lse = {m, log2_of_sum(s) - fmaf(m, kLog2e, -ms)};  // minus what ms lost to rounding
     if (live && j == 0) {
-        lse_out[r] = lse;
+        lse_out[r] = lse.value();
         const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
         const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
         int lab = -1;
@@ -586,7 +620,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_small(
             lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
-            const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
+            const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
             lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
         } else if (grads_skipped) {
             grads_skipped[r] = make_float2(0.f, 0.f);
@@ -614,9 +648,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     float s = 0.f;
     for (int v = lane; v < V; v += 64) s += fast_exp2(fmaf(Elem<T>::to_f32(row[v]), kLog2e, -ms));
     s = group_allreduce<64, OpSum>(s);
-    const float lse = fmaf(fast_log2(s), kLn2, m);
+    const Lse lse = {m, log2_of_sum(s) - fmaf(m, kLog2e, -ms)};  // minus what ms lost to rounding
     if (lane == 0) {
-        lse_out[r] = lse;
+        lse_out[r] = lse.value();
         const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
         const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
         int lab = -1;
@@ -624,7 +658,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
             lab = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
-            const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : lse;
+            const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
             lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
         } else if (grads_skipped) {
             grads_skipped[r] = make_float2(0.f, 0.f);
@@ -652,7 +686,7 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
         const T* row = x + r * (i64)V;
         const float xb = Elem<T>::to_f32(row[blank]);
         const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-        lp[dst] = make_lp(xb, xl, 0.f, lab >= 0, seqmode + ri.n);
+        lp[dst] = make_lp(xb, xl, Lse{0.f, 0.f}, lab >= 0, seqmode + ri.n);
     } else if (grads_skipped) {
         grads_skipped[r] = make_float2(0.f, 0.f);
     }

@@ -566,6 +566,21 @@ def test_reduction_is_nan_when_a_sequence_is_skipped():
     assert torch.isnan(costs).all() and torch.isnan(st.reduced).all()
 
 
+def test_peaked_rows_keep_the_absolute_accuracy_of_small_costs():
+    """Logits of large magnitude over a tiny vocabulary: most rows are one-hot, log-probabilities of
+    the likely entries are ~1e-6 below zero and a cost can be a few hundredths of a nat while the
+    row maxima are ~25.  The log-probabilities must not inherit the rounding of the fp32
+    log-sum-exp (half an ulp of 25 per cell)."""
+    rng = np.random.default_rng(4242)
+    for case in range(60):
+        N = 12
+        lx = rng.integers(1, 40, N)
+        ly = rng.integers(0, 30, N)
+        dtype = ["f32", "bf16", "f64"][case % 3]
+        b = make_batch(lx, ly, 2, seed=int(rng.integers(1 << 30)), sigma=12.0, dtype=dtype, blank=case % 2)
+        check_case(b, True, "2d", dtype=dtype, seed=case)
+
+
 # ----------------------------------------------------------------------------- randomised sweep
 @pytest.mark.parametrize("seed", range(12))
 def test_random_shapes_against_oracle(seed):
