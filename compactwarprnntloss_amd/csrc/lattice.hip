@@ -877,7 +877,9 @@ __device__ __forceinline__ bool fill_slot(const int* __restrict__ lx, const int*
         double fa = a + (double)cell.l_blank;
         double fb = b00;
         double ratio = fabs(fa - fb) / fabs(fmax(fa, fb));
-        if (ratio > 1e-3) {
+        // the reference's rule is relative only; a likelihood within rounding of 1 (both logarithms
+        // ~1e-7) has no meaningful relative difference, hence the absolute floor
+        if (ratio > 1e-3 && fabs(fa - fb) > 1e-5) {
             atomicOr(status, CWR_FLAG_FB_MISMATCH);
             fb = (fa + fb) * 0.5;
         }

@@ -65,9 +65,10 @@ enum cwr_flag {
     CWR_FLAG_ROWS_MISMATCH = 1, /* sum lx*(ly+1) != R */
     CWR_FLAG_BAD_LENGTH = 2,    /* some lx <= 0 or ly < 0 (that sequence is skipped, cost = NaN) */
     CWR_FLAG_BAD_LABEL = 4,     /* a label outside [0, V) was met (treated as "no label") */
-    CWR_FLAG_FB_MISMATCH = 8,   /* forward and backward likelihood differ by > 0.1 % for some
-                                   sequence; the cost is their mean, as in the reference
-                                   (cwarp_cuda_rnnt_kernel.cu:356-364, which prints instead) */
+    CWR_FLAG_FB_MISMATCH = 8,   /* forward and backward log-likelihood differ by > 0.1 % (and by
+                                   more than 1e-5, so that a likelihood within rounding of 1 does
+                                   not count) for some sequence; the cost is their mean, as in the
+                                   reference (cwarp_cuda_rnnt_kernel.cu:356-364, which prints) */
     CWR_FLAG_U_TOO_LARGE = 16,  /* some ly exceeds the max_u given to the call */
     CWR_FLAG_INTERNAL = 32      /* a bounded wait inside a kernel ran out (results are invalid) */
 };

@@ -581,6 +581,18 @@ def test_peaked_rows_keep_the_absolute_accuracy_of_small_costs():
         check_case(b, True, "2d", dtype=dtype, seed=case)
 
 
+def test_near_certain_sequences_do_not_flag_a_mismatch():
+    """A blank that is all but certain and sequences without labels: costs of ~1e-7, where the
+    reference's relative forward/backward rule (cwarp_cuda_rnnt_kernel.cu:353-366) compares two
+    roundings of zero.  No flag, costs within 1e-6 of the oracle."""
+    b = make_batch([52, 46, 10, 2], [0, 80, 56, 0], 24, seed=3, dtype="bf16", blank=14)
+    x = b["x"].float()
+    x[:, 14] += 25.0
+    b["x"] = x.to(torch.bfloat16)
+    b["x_ref"] = b["x"].double().numpy()
+    check_case(b, True, "2d", dtype="bf16")
+
+
 # ----------------------------------------------------------------------------- randomised sweep
 @pytest.mark.parametrize("seed", range(12))
 def test_random_shapes_against_oracle(seed):
