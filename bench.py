@@ -143,11 +143,16 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # events between the steps (recorded, never waited on inside the timed region) give the spread
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for k in range(args.steps):
         step()
+        marks[k + 1].record()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_step = sorted(marks[k].elapsed_time(marks[k + 1]) for k in range(args.steps))
 
     # per-call timing with events on the stream the kernels run on (torch's current stream)
     xd = x.detach()
@@ -189,6 +194,8 @@ def main():
         "config": {"workload": WORKLOADS[args.config], "N": N, "R": R, "V": V,
                    "algorithmic_bytes_per_step": bytes_step, "entry": "cwarp_rnnt.transducer_loss"},
         "pct_of_hbm_peak": round(100.0 * bytes_step / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "step_ms": {"median": round(per_step[len(per_step) // 2], 4), "min": round(per_step[0], 4),
+                    "max": round(per_step[-1], 4)},
         "breakdown_ms": {"forward_call": round(fwd_ms, 4), "backward_call": round(bwd_ms, 4),
                          "forward_nograd_call": round(nograd_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": "k_grad (cwr_backward)", "achieved": round(achieved, 1),
