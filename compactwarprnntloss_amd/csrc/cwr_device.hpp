@@ -163,6 +163,14 @@ template <> struct Elem<double> {
     static __device__ __forceinline__ double from_f32(float v) { return (double)v; }
 };
 
+// 16-byte store of data that nothing on the GPU reads again soon: non-temporal AND system scope.
+// The compiler's non-temporal store sets only the first of the two; with both the (R,V) gradient
+// stream runs about 3 % faster on MI355X (395 -> 383 us for 1.28 GB read + 1.28 GB written).
+typedef int v4i_store_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_streaming_16(void* p, v4i_store_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(p), "v"(v) : "memory");
+}
+
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PackT { T e[VEC]; };
 
 template <typename T, int VEC>

@@ -86,7 +86,7 @@ __device__ __forceinline__ void st_stream(T* p, const PackT<T, VEC>& v) {
     if constexpr (sizeof(T) * VEC == 16) {
         v4i r;
         __builtin_memcpy(&r, &v, 16);
-        __builtin_nontemporal_store(r, reinterpret_cast<v4i*>(p));
+        store_streaming_16(p, r);
     } else {
         *reinterpret_cast<PackT<T, VEC>*>(p) = v;
     }

@@ -23,7 +23,7 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 template <> struct Unit<v4i_t> {
     static __device__ __forceinline__ v4i_t zero() { v4i_t z = {0, 0, 0, 0}; return z; }
     static __device__ __forceinline__ v4i_t load(const v4i_t* p) { return __builtin_nontemporal_load(p); }
-    static __device__ __forceinline__ void store(v4i_t* p, v4i_t v) { __builtin_nontemporal_store(v, p); }
+    static __device__ __forceinline__ void store(v4i_t* p, v4i_t v) { store_streaming_16(p, v); }
 };
 
 // grid: x = (label position u, block of 4 chunks of 64 units), y = frame t, z = sequence n (relative

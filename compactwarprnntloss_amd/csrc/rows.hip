@@ -29,7 +29,7 @@ __device__ __forceinline__ v4i load_raw(const void* p) {
 template <bool NT>
 __device__ __forceinline__ void store_raw(void* p, v4i v) {
     v4i* q = static_cast<v4i*>(p);
-    if (NT) __builtin_nontemporal_store(v, q); else *q = v;
+    if (NT) store_streaming_16(q, v); else *q = v;
 }
 
 // 16-byte pack <-> VEC fp32 values
