@@ -4,7 +4,9 @@ The reference repository holds no golden vectors and cannot be built or run with
 fixtures are produced by the float64 oracle (oracle/rnnt_oracle.py), which tests/test_oracle_pins.py
 pins against brute-force path enumeration, closed forms, finite differences and autograd.  Each
 file stores inputs (x, lx, ly, y, blank, mode, grad_out) and expected outputs (costs, G, grad,
-int32 row offsets).  Run from the repository root:  python tests/golden/make_golden.py
+int32 row offsets).  The join_*.npz files hold the compact joiner front instead: inputs (f, g, lx,
+ly, act, dh) and expected outputs (h, df, dg) from the oracle's join_rows / join_rows_backward.
+Run from the repository root:  python tests/golden/make_golden.py
 """
 import os
 import sys
@@ -53,5 +55,29 @@ def main():
         print(name, "R =", R, "costs", np.round(out["costs"], 4))
 
 
+JOIN_CASES = [
+    # name, lx, ly, H, activation, seed, padding of (T, U+1) beyond the longest sequence
+    ("join_tanh", [5, 1, 7, 3], [2, 4, 0, 6], 24, "tanh", 7, (1, 2)),
+    ("join_sum", [3, 6], [5, 1], 10, "none", 8, (0, 0)),
+]
+
+
+def main_join():
+    for name, lx, ly, H, act, seed, (tp, up) in JOIN_CASES:
+        rng = np.random.default_rng(seed)
+        lx = np.asarray(lx, dtype=np.int32)
+        ly = np.asarray(ly, dtype=np.int32)
+        N = len(lx)
+        f = rng.standard_normal((N, int(lx.max()) + tp, H)).astype(np.float32)
+        g = rng.standard_normal((N, int(ly.max()) + 1 + up, H)).astype(np.float32)
+        h = orc.join_rows(f, g, lx, ly, act)
+        dh = rng.standard_normal(h.shape).astype(np.float32)
+        df, dg = orc.join_rows_backward(dh, f, g, lx, ly, act)
+        np.savez_compressed(os.path.join(HERE, name + ".npz"), f=f, g=g, lx=lx, ly=ly, act=np.array(act), dh=dh,
+                            h=h, df=df, dg=dg)
+        print(name, "rows =", h.shape[0], "H =", H)
+
+
 if __name__ == "__main__":
+    main_join()
     main()

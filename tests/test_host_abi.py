@@ -201,8 +201,15 @@ def test_golden_fixtures_match_the_oracle():
     """The committed fixtures (written by tests/golden/make_golden.py from the oracle) still
     reproduce: guards the oracle against silent edits."""
     gdir = os.path.join(ROOT, "tests", "golden")
-    files = sorted(f for f in os.listdir(gdir) if f.endswith(".npz"))
+    files = sorted(f for f in os.listdir(gdir) if f.endswith(".npz") and not f.startswith("join_"))
     assert files, "no golden fixtures"
+    for f in sorted(f for f in os.listdir(gdir) if f.startswith("join_") and f.endswith(".npz")):
+        z = np.load(os.path.join(gdir, f))
+        act = str(z["act"])
+        np.testing.assert_allclose(orc.join_rows(z["f"], z["g"], z["lx"], z["ly"], act), z["h"], rtol=1e-14)
+        df, dg = orc.join_rows_backward(z["dh"], z["f"], z["g"], z["lx"], z["ly"], act)
+        np.testing.assert_allclose(df, z["df"], rtol=1e-12, atol=1e-15)
+        np.testing.assert_allclose(dg, z["dg"], rtol=1e-12, atol=1e-15)
     for f in files:
         z = np.load(os.path.join(gdir, f))
         mode = str(z["mode"])

@@ -172,3 +172,24 @@ def test_join_and_pack_random_batches(seed):
     acc = torch.float64 if dtype == "f64" else torch.float32
     z = (fd.to(acc)[:, :, None, :] + gd.to(acc)[:, None, :, :]).to(fd.dtype).contiguous()
     assert torch.equal(pkg.pack_padded(z, lxd, lyd), h)
+
+
+def _join_fixtures():
+    import os
+    gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    return sorted(os.path.join(gdir, f) for f in os.listdir(gdir) if f.startswith("join_") and f.endswith(".npz"))
+
+
+@pytest.mark.parametrize("path", _join_fixtures(), ids=lambda p: p.split("/")[-1][:-4])
+def test_join_against_golden_fixtures(path):
+    pkg = _pkg()
+    z = np.load(path)
+    act = str(z["act"])
+    f = torch.from_numpy(z["f"]).to(DEV).requires_grad_(True)
+    g = torch.from_numpy(z["g"]).to(DEV).requires_grad_(True)
+    lx, ly = torch.from_numpy(z["lx"]).to(DEV), torch.from_numpy(z["ly"]).to(DEV)
+    h = pkg.compact_join(f, g, lx, ly, None if act == "none" else act)
+    np.testing.assert_allclose(h.detach().cpu().numpy(), z["h"], rtol=3e-7, atol=6e-7)
+    h.backward(torch.from_numpy(z["dh"]).to(DEV))
+    np.testing.assert_allclose(f.grad.cpu().numpy(), z["df"], rtol=1e-6, atol=2e-5)
+    np.testing.assert_allclose(g.grad.cpu().numpy(), z["dg"], rtol=1e-6, atol=2e-5)
