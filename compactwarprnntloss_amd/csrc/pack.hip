@@ -5,7 +5,7 @@
 // T_i x (U_i+1) sub-lattice are selected, in the order of test/test.py:44-46.  Rows move in
 // 16-byte units (or element-sized units when rows are not 16-byte multiples).  pack walks the
 // compact rows (k_pack_rows); unpack has to write every padded element and takes one workgroup
-// per 256 units of one PADDED row, whose (n, t, u) comes straight from the grid (k_repack).
+// per 256 units of one PADDED row, whose (n, t, u) comes straight from the grid (k_unpack).
 //   pack:   compact[row_off[n] + t*(U_n+1) + u] = padded[n][t][u]      for t < T_n, u <= U_n
 //   unpack: padded[n][t][u] = the same compact row, or zeros outside the sub-lattice (this is the
 //           backward of pack: every element of the padded gradient is written, no memset pass)
@@ -28,37 +28,29 @@ template <> struct Unit<v4i_t> {
 
 // grid: x = (label position u, block of 4 chunks of 64 units), y = frame t, z = sequence n (relative
 // to n0), so that no wave needs a 64-bit division and consecutive workgroups walk memory in order.
-template <typename U, bool UNPACK>
-__global__ __launch_bounds__(256) void k_repack(const U* __restrict__ src, U* __restrict__ dst,
+template <typename U>
+__global__ __launch_bounds__(256) void k_unpack(const U* __restrict__ src, U* __restrict__ dst,
                                                  const int* __restrict__ lx, const int* __restrict__ ly,
                                                  const i64* __restrict__ row_off, int n0, int T_pad, int Up_pad,
-                                                 i64 units_per_row, unsigned cblocks, i64 R,
-                                                 int* __restrict__ status) {
+                                                 i64 units_per_row, unsigned cblocks, i64 R) {
     const int lane = threadIdx.x & 63;
     const int n = n0 + (int)blockIdx.z;
     const int t = (int)blockIdx.y;
     const unsigned u = cblocks == 1 ? blockIdx.x : blockIdx.x / cblocks;
     const unsigned cb = blockIdx.x - u * cblocks;
     const int T = lx[n], Ul = ly[n];
-    if (status && t == 0 && blockIdx.x == 0 && threadIdx.x == 0 && (T > T_pad || Ul + 1 > Up_pad))
-        atomicOr(status, CWR_FLAG_BAD_LENGTH);  // part of this sequence lies outside the padded array
     bool valid = T > 0 && Ul >= 0 && t < T && (int)u <= Ul;
     i64 crow = 0;
     if (valid) {
         crow = row_off[n] + (i64)t * ((i64)Ul + 1) + u;
         if (crow >= R) valid = false;  // lengths that do not add up to R: flagged by the offsets pass
     }
-    if (!UNPACK && !valid) return;
     const i64 unit = ((i64)cb * 4 + (threadIdx.x >> 6)) * 64 + lane;
     if (unit >= units_per_row) return;
     const i64 prow = ((i64)n * T_pad + t) * Up_pad + u;
-    if (UNPACK) {
-        U v = Unit<U>::zero();
-        if (valid) v = Unit<U>::load(src + crow * units_per_row + unit);
-        Unit<U>::store(dst + prow * units_per_row + unit, v);
-    } else {
-        Unit<U>::store(dst + crow * units_per_row + unit, Unit<U>::load(src + prow * units_per_row + unit));
-    }
+    U v = Unit<U>::zero();
+    if (valid) v = Unit<U>::load(src + crow * units_per_row + unit);
+    Unit<U>::store(dst + prow * units_per_row + unit, v);
 }
 
 // pack, walking the COMPACT rows instead: a wave takes `rpw` consecutive rows (about 4 KiB), decodes
@@ -121,9 +113,9 @@ static int repack_as(const void* src, void* dst, const int* lx, const int* ly, c
     for (i64 n0 = 0; n0 < N; n0 += 65535) {
         const i64 nz = N - n0 < 65535 ? N - n0 : 65535;
         dim3 grid((unsigned)(Up_pad * cblocks), (unsigned)T_pad, (unsigned)nz);
-        hipLaunchKernelGGL((k_repack<U, true>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
+        hipLaunchKernelGGL((k_unpack<U>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
                            static_cast<U*>(dst), lx, ly, row_off, (int)n0, (int)T_pad, (int)Up_pad,
-                           units_per_row, (unsigned)cblocks, R, status);
+                           units_per_row, (unsigned)cblocks, R);
         int rc = check_launch();
         if (rc != CWR_OK) return rc;
     }
