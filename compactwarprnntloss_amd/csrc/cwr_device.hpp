@@ -119,18 +119,6 @@ __device__ __forceinline__ i64 wave_inclusive_scan(i64 v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// log2(2^a + 2^b) = max + log2(1 + 2^-|a-b|): the form of cwarp_cuda_rnnt_kernel.cu:22-29 in
-// base 2, so that it maps onto the hardware exp2/log2 units without scaling multiplies.
-// The running values are kept in fp64 (a lattice of ~2000 steps reaches magnitudes of several
-// thousand, where an fp32 ulp is already 2e-4); the correction term, at most 1, is evaluated in
-// fp32 from the fp32-rounded difference.
-__device__ __forceinline__ double log2_sum_exp2(double a, double b) {
-    double mx = fmax(a, b);
-    float d = (float)(a - b);
-    float e = fast_exp2(-fabsf(d));
-    return mx + (double)fast_log2(1.0f + e);
-}
-
 // ---------------------------------------------------------------------------------------------
 // element packs: VEC consecutive elements moved with one 16-byte access, computed on as fp32
 // ---------------------------------------------------------------------------------------------
@@ -172,20 +160,6 @@ __device__ __forceinline__ void store_streaming_16(void* p, v4i_store_t v) {
 }
 
 template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PackT { T e[VEC]; };
-
-template <typename T, int VEC>
-__device__ __forceinline__ void load_pack(const T* __restrict__ p, float (&out)[VEC]) {
-    PackT<T, VEC> raw = *reinterpret_cast<const PackT<T, VEC>*>(p);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) out[i] = Elem<T>::to_f32(raw.e[i]);
-}
-template <typename T, int VEC>
-__device__ __forceinline__ void store_pack(T* __restrict__ p, const float (&in)[VEC]) {
-    PackT<T, VEC> raw;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) raw.e[i] = Elem<T>::from_f32(in[i]);
-    *reinterpret_cast<PackT<T, VEC>*>(p) = raw;
-}
 
 // ---------------------------------------------------------------------------------------------
 // layouts

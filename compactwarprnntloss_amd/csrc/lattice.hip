@@ -46,10 +46,6 @@ __device__ __forceinline__ void buf_store_d(__amdgpu_buffer_rsrc_t r, int voff, 
     v.y = __double2hiint(x);
     __builtin_amdgcn_raw_buffer_store_b64(v, r, voff, soff, 0);
 }
-__device__ __forceinline__ void buf_store_zero8(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    v2i z = {0, 0};
-    __builtin_amdgcn_raw_buffer_store_b64(z, r, voff, soff, 0);
-}
 __device__ __forceinline__ void buf_store_zero16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     v4i z = {0, 0, 0, 0};
     __builtin_amdgcn_raw_buffer_store_b128(z, r, voff, soff, 0);
@@ -236,23 +232,6 @@ __device__ __forceinline__ void settle_loads() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
     __builtin_amdgcn_sched_barrier(0);
 }
-
-__device__ __forceinline__ int exponent_of(double x) {
-    return x == 0.0 ? kNoExp : __builtin_amdgcn_frexp_exp(x);
-}
-// Maximum over the wave.  `old` = INT_MIN is the identity of max, which lets the compiler fold
-// each cross-lane move into the v_max_i32 that consumes it.
-__device__ __forceinline__ int wave_max_i32(int v) {
-    constexpr int kMin = (int)0x80000000;
-    v = max(v, dpp_i32<DPP_QUAD_XOR1>(kMin, v));
-    v = max(v, dpp_i32<DPP_QUAD_XOR2>(kMin, v));
-    v = max(v, dpp_i32<DPP_ROW_HALF_MIRROR>(kMin, v));
-    v = max(v, dpp_i32<DPP_ROW_MIRROR>(kMin, v));
-    v = max(v, dpp_i32<DPP_ROW_BCAST15, 0xA>(kMin, v));
-    v = max(v, dpp_i32<DPP_ROW_BCAST31, 0xC>(kMin, v));
-    return __builtin_amdgcn_readlane(v, 63);
-}
-__device__ __forceinline__ double exp2_f64(float x) { return (double)fast_exp2(x); }
 
 // Both walks share one shape.  A ring of kPF registers holds the gathered records of the next
 // kPF steps; step j issues the load that refills ring[j] and prepares the NEXT step's two
@@ -552,6 +531,9 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
             const float2 cn = buf_load_f2(r_cell, vo_l, (mi + dq * kPF) * p16);
             const double old = HAS_IN ? readlane_f64(e_lane, j) : nbr;
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(old, pass) : dpp_f64<DPP_WAVE_SHR1>(old, pass);
+            // log2(2^own + 2^nbr) = max + log2(1 + 2^-|own-nbr|): the form of
+            // cwarp_cuda_rnnt_kernel.cu:22-29 in base 2; the running values are fp64, the correction
+            // term (at most 1) comes from the fp32 exp2 / log2 units
             const double mx = fmax(own, nbr);
             const float d = (float)(own - nbr);
             const double l = (double)fast_log2(1.0f + fast_exp2(-fabsf(d)));
