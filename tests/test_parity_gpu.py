@@ -620,3 +620,45 @@ def test_random_shapes_against_oracle(seed):
         except AssertionError as err:
             raise AssertionError(f"seed {seed} case {case}: N={N} lx={lx.tolist()} ly={ly.tolist()} V={V} "
                                  f"{dtype} fused={fused} blank={blank} sigma={sigma} labels={labels}\n{err}")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_hard_regimes_against_oracle(seed):
+    """Twenty-five random batches per seed from the regimes that leave the comfortable number range:
+    steep logits (sigma 20 to 80), one column shifted far from the others, -inf entries no label
+    uses, many strips (up to 720 labels: the sequential walk) and long sequences (up to 900 frames)."""
+    rng = np.random.default_rng(31000 + seed)
+    for case in range(25):
+        N = int(rng.integers(1, 5))
+        kind = str(rng.choice(["steep", "columns", "mask", "strips", "longt"]))
+        lx = rng.integers(1, 60, N)
+        ly = rng.integers(0, 90, N)
+        V = int(rng.choice([3, 8, 24, 64, 130]))
+        fused = bool(rng.integers(0, 2))
+        sigma = float(rng.choice([20.0, 40.0, 80.0])) if kind == "steep" else 1.0
+        if kind == "strips":
+            ly, lx, V = rng.integers(60, 720, N), rng.integers(1, 50, N), int(rng.choice([3, 8]))
+        if kind == "longt":
+            lx, ly, V = rng.integers(300, 900, N), rng.integers(0, 70, N), int(rng.choice([3, 8]))
+        dtype = str(rng.choice(["f32", "f32", "f16", "bf16", "f64"]))
+        blank = int(rng.integers(0, V))
+        b = make_batch(lx, ly, V, seed=int(rng.integers(1 << 30)), sigma=sigma, dtype=dtype, blank=blank,
+                       normalised=not fused)
+        if kind in ("columns", "mask"):
+            x = b["x"].clone().float()
+            if kind == "columns" and fused:
+                x[:, blank] += float(rng.choice([-30.0, -50.0, 25.0]))
+            elif kind == "columns":
+                x[:, blank] = float(rng.choice([-10.0, -30.0, -45.0, -62.0]))
+            else:
+                used = set(np.unique(b["yp"]).tolist()) | {blank}
+                free = [v for v in range(V) if v not in used]
+                if free:
+                    x[:, free[: max(1, len(free) // 2)]] = -float("inf")
+            b["x"] = x.to(TORCH_DT[dtype])
+            b["x_ref"] = b["x"].double().numpy()
+        try:
+            check_case(b, fused, str(rng.choice(["2d", "1d"])), dtype=dtype, seed=case)
+        except AssertionError as err:
+            raise AssertionError(f"seed {seed} case {case} ({kind}): N={N} lx={lx.tolist()} ly={ly.tolist()} V={V} "
+                                 f"{dtype} fused={fused} blank={blank} sigma={sigma}\n{err}")
