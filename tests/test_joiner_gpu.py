@@ -193,3 +193,29 @@ def test_join_against_golden_fixtures(path):
     h.backward(torch.from_numpy(z["dh"]).to(DEV))
     np.testing.assert_allclose(f.grad.cpu().numpy(), z["df"], rtol=1e-6, atol=2e-5)
     np.testing.assert_allclose(g.grad.cpu().numpy(), z["dg"], rtol=1e-6, atol=2e-5)
+
+
+def test_joiner_and_loss_train_a_tiny_model():
+    """End to end: a few Adam steps on random encoder / predictor features must drive the loss
+    down (joiner front, library GEMMs, fused loss and all three backward passes together)."""
+    pkg = _pkg()
+    torch.manual_seed(1)
+    lx, ly = np.array([14, 9, 20, 6], dtype=np.int32), np.array([4, 6, 3, 0], dtype=np.int32)
+    N, E, P, J, V = 4, 16, 12, 32, 11
+    enc = torch.randn(N, int(lx.max()), E, device=DEV)
+    pred = torch.randn(N, int(ly.max()) + 1, P, device=DEV)
+    y = torch.randint(1, V, (N, int(ly.max())), dtype=torch.int32, device=DEV)
+    lxd, lyd = torch.from_numpy(lx).to(DEV), torch.from_numpy(ly).to(DEV)
+    R = int((lx.astype(np.int64) * (ly + 1)).sum())
+    joiner = pkg.CompactJoiner(E, P, J, V).to(DEV)
+    opt = torch.optim.Adam(joiner.parameters(), lr=3e-2)
+    losses = []
+    for _ in range(40):
+        opt.zero_grad()
+        loss = pkg.transducer_loss(joiner(enc, pred, lxd, lyd, total_rows=R), lxd, y, lyd, 0, "mean",
+                                   fused_log_softmax=True)
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(np.isfinite(losses))
+    assert losses[-1] < 0.5 * losses[0], losses[::8]
