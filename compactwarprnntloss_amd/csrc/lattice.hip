@@ -353,8 +353,23 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     settle_loads();
     int k0 = 0;
     for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
-        if (HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
-        if (HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+        // The two counters and (speculatively) the incoming entries in ONE LDS round trip: LDS
+        // serves a wave's requests in order, so entries read after a counter that already shows them
+        // produced are the produced ones.  Only a counter that falls short sends the wave polling.
+        double2 en_first = make_double2(0.0, 0.0);
+        {
+            int prod = 0x7fffffff, cons = 0x7fffffff;
+            if (HAS_IN) prod = __hip_atomic_load(rin.produced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (HAS_OUT) cons = __hip_atomic_load(rout.consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            keep_order();
+            if (HAS_IN) en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+            if (HAS_IN && prod < k0 + kPF + in_shift) {
+                wait_at_least(rin.produced, k0 + kPF + in_shift, status);
+                keep_order();
+                en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+            }
+            if (HAS_OUT && cons < k0 + kPF - kRing - out_shift) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+        }
         keep_order();
         // Renew the scales.  True magnitude (binary exponent minus scale) of what the lane holds,
         // of what it will hand over and of what its neighbour will hand over next:
@@ -365,7 +380,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
-            const double2 en = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+            const double2 en = en_first;
             double ev = en.x;
             if (BETA) {
                 ev *= (double)edge;
@@ -392,15 +407,19 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             t = max(t, dpp_i32<DPP_ROW_SHL + 2>(kNoExp, t));
             t = max(t, dpp_i32<DPP_ROW_SHL + 4>(kNoExp, t));
             t = max(t, dpp_i32<DPP_ROW_SHL + 8>(kNoExp, t));
-            const int next_row = __shfl(t, (lane | 15) + 1 > 63 ? lane : (lane | 15) + 1);
-            if (lane < 48) t = max(t, next_row);
+            // lane 0 of a row now holds the row's maximum: three scalar reads instead of a trip
+            // through the LDS crossbar
+            const int r1 = __builtin_amdgcn_readlane(t, 16), r2 = __builtin_amdgcn_readlane(t, 32),
+                      r3 = __builtin_amdgcn_readlane(t, 48);
+            const int next_row = lane < 16 ? r1 : (lane < 32 ? r2 : (lane < 48 ? r3 : kNoExp));
+            t = max(t, next_row);
         } else {
             t = max(t, dpp_i32<DPP_ROW_SHR + 1>(kNoExp, t));
             t = max(t, dpp_i32<DPP_ROW_SHR + 2>(kNoExp, t));
             t = max(t, dpp_i32<DPP_ROW_SHR + 4>(kNoExp, t));
             t = max(t, dpp_i32<DPP_ROW_SHR + 8>(kNoExp, t));
-            const int prev_row = __shfl(t, lane < 16 ? lane : (lane & ~15) - 1);
-            if (lane >= 16) t = max(t, prev_row);
+            // lane 15 of a row now holds the row's maximum: one broadcast into the next row
+            t = max(t, dpp_i32<DPP_ROW_BCAST15, 0xE>(kNoExp, t));
         }
         const bool empty = t <= kNoExp / 2;
         int Cn = empty ? C : kLinTarget - t;
