@@ -200,6 +200,8 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 constexpr int kRing = 256;             // entries of an LDS boundary ring (a multiple of kPF)
 constexpr int kSpinLimit = 1 << 22;    // polls after which a waiting wave gives up
 constexpr int kNoExp = -(1 << 20);     // "exponent" of zero
+constexpr int kDppMin = (int)0x80000000;  // what a lane without a DPP source contributes to a maximum: with the
+                                          // identity of max there, the move folds into the v_max_i32 that uses it
 
 struct Ring {
     double2* slots;  // LDS, kRing entries (value, exponent C of the producer) + a dummy area behind
@@ -376,7 +378,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         const int t_own = own != 0.0 ? __builtin_amdgcn_frexp_exp(own) - C : kNoExp;
         const int t_pass = pass != 0.0 ? __builtin_amdgcn_frexp_exp(pass) - C : kNoExp;
         int t = max(max(t_own, t_pass),
-                    BETA ? dpp_i32<DPP_WAVE_SHL1>(kNoExp, t_pass) : dpp_i32<DPP_WAVE_SHR1>(kNoExp, t_pass));
+                    BETA ? dpp_i32<DPP_WAVE_SHL1>(kDppMin, t_pass) : dpp_i32<DPP_WAVE_SHR1>(kDppMin, t_pass));
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
@@ -392,10 +394,10 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             e_lane = ok ? ev : 0.0;
             // the largest of the kPF entries (they sit in every row of 16 lanes), for the edge lane
             int te = ok ? __builtin_amdgcn_frexp_exp(ev) - cp : kNoExp;
-            te = max(te, dpp_i32<DPP_QUAD_XOR1>(kNoExp, te));
-            te = max(te, dpp_i32<DPP_QUAD_XOR2>(kNoExp, te));
-            te = max(te, dpp_i32<DPP_ROW_HALF_MIRROR>(kNoExp, te));
-            te = max(te, dpp_i32<DPP_ROW_MIRROR>(kNoExp, te));
+            te = max(te, dpp_i32<DPP_QUAD_XOR1>(kDppMin, te));
+            te = max(te, dpp_i32<DPP_QUAD_XOR2>(kDppMin, te));
+            te = max(te, dpp_i32<DPP_ROW_HALF_MIRROR>(kDppMin, te));
+            te = max(te, dpp_i32<DPP_ROW_MIRROR>(kDppMin, te));
             if (lane == in_lane) t = max(t, te);
         }
         // Whatever reaches a lane during this block was, at its start, in one of the kPF lanes the
@@ -403,10 +405,10 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         // magnitude over that window, so that nothing arriving can exceed 2^(kLinTarget + kPF*
         // (kLinMax+1)).  Window used: the lanes before it in its row of 16 and the whole row before.
         if (BETA) {
-            t = max(t, dpp_i32<DPP_ROW_SHL + 1>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHL + 2>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHL + 4>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHL + 8>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 1>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 2>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 4>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHL + 8>(kDppMin, t));
             // lane 0 of a row now holds the row's maximum: three scalar reads instead of a trip
             // through the LDS crossbar
             const int r1 = __builtin_amdgcn_readlane(t, 16), r2 = __builtin_amdgcn_readlane(t, 32),
@@ -414,12 +416,12 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             const int next_row = lane < 16 ? r1 : (lane < 32 ? r2 : (lane < 48 ? r3 : kNoExp));
             t = max(t, next_row);
         } else {
-            t = max(t, dpp_i32<DPP_ROW_SHR + 1>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHR + 2>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHR + 4>(kNoExp, t));
-            t = max(t, dpp_i32<DPP_ROW_SHR + 8>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 1>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 2>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 4>(kDppMin, t));
+            t = max(t, dpp_i32<DPP_ROW_SHR + 8>(kDppMin, t));
             // lane 15 of a row now holds the row's maximum: one broadcast into the next row
-            t = max(t, dpp_i32<DPP_ROW_BCAST15, 0xE>(kNoExp, t));
+            t = max(t, dpp_i32<DPP_ROW_BCAST15, 0xE>(kDppMin, t));
         }
         const bool empty = t <= kNoExp / 2;
         int Cn = empty ? C : kLinTarget - t;
@@ -435,7 +437,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         d = C - (BETA ? dpp_i32<DPP_WAVE_SHL1>(C, C) : dpp_i32<DPP_WAVE_SHR1>(C, C));
         if (lane >= nl) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
         if (HAS_IN) e_lane = __builtin_ldexp(e_lane, __builtin_amdgcn_readlane(C, in_lane) - cp);
-        buf_store_i32(r_sc, vo_sc, blk * p4, C);
+        buf_store_i32(r_sc, vo_sc, __builtin_amdgcn_readfirstlane(blk * p4), C);  // wave-uniform, and said so
         const double Cd = (double)__builtin_amdgcn_readlane(C, out_lane);
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
