@@ -893,13 +893,17 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_flat(
     const GradOut grad_costs, T* __restrict__ gx) {
     constexpr int VEC = Elem<T>::VEC;
     const int lane = threadIdx.x & 63;
-    const i64 wave = wave_first_row<true>(1);  // global wave index
-    const i64 r = wave / chunks_per_row;
-    if (r >= R) return;
-    const int pack = (int)(wave - r * chunks_per_row) * 64 + lane;
-    const i64 at = r * (i64)V + (i64)pack * VEC;
+    // global wave index = chunk of 64 packs in the flat tensor; the host keeps their number below 2^31
+    const unsigned wave = (unsigned)wave_first_row<true>(1);
+    if ((i64)wave >= R * chunks_per_row) return;
+    // rows are whole numbers of chunks, so the address needs no row: the load goes out first and the
+    // (32-bit, branch-free) division that finds the row runs under it
+    const i64 at = ((i64)wave * 64 + lane) * VEC;
     v4i in = {0, 0, 0, 0};
     if (FUSED) in = load_raw<NT>(x + at);
+    const unsigned ur = wave / (unsigned)chunks_per_row;
+    const i64 r = ur;
+    const int pack = (int)(wave - ur * (unsigned)chunks_per_row) * 64 + lane;
     const RowCoef rc = row_coef<FUSED>(r, N, rowinfo, grads, lse, grad_costs);
     store_raw<NT>(gx + at, grad_pack<T, FUSED>(in, rc, pack, blank, V));
 }
@@ -1100,7 +1104,7 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
     int lpr = 0, k = 0;
     if (packed_ok<T>(grad_x, b.V) && (!FUSED || packed_ok<T>(b.x, b.V))) {
         const int NV = b.V / Elem<T>::VEC;
-        if (NV % 64 == 0) {
+        if (NV % 64 == 0 && b.R * (i64)(NV / 64) < 0x7fffffffLL) {  // (2^31 chunks of 1 KiB would be 2 TiB)
             const int ch = NV / 64;
             hipLaunchKernelGGL((k_grad_flat<T, FUSED, kGradNT>), dim3((blocks_for_waves(b.R * ch) + 7u) & ~7u),
                                dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ch, ri, g2,
