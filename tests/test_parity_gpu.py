@@ -442,6 +442,16 @@ def test_rows_beyond_two_to_the_31_elements(fused):
         assert float(tail.abs().max()) < 2e-2   # 1024 fp16-rounded entries per row
 
 
+@pytest.mark.parametrize("fused,V", [(True, 16), (False, 64)])
+def test_thousands_of_short_sequences(fused, V):
+    """3000 sequences of a few cells each: the offsets scan in chunks of 64, one lattice workgroup
+    per sequence and direction, and every per-sequence lookup far beyond the in-register tables."""
+    rng = np.random.default_rng(6)
+    N = 3000
+    b = make_batch(rng.integers(1, 7, N), rng.integers(0, 4, N), V, seed=N, normalised=not fused)
+    check_case(b, fused, "1d", seed=1)
+
+
 # ----------------------------------------------------------------------------- number systems of the lattice walk
 def _walk_modes(st):
     """Per-sequence walk-mode words of a forward call (workspace section 4)."""
