@@ -204,8 +204,9 @@ constexpr int kDppMin = (int)0x80000000;  // what a lane without a DPP source co
                                           // identity of max there, the move folds into the v_max_i32 that uses it
 
 struct Ring {
-    double2* slots;  // LDS, kRing entries (value, exponent C of the producer) + a dummy area behind
-                     // them for the lanes that hold no edge
+    double* slots;   // LDS, kRing values + a dummy area behind them for the lanes that hold no edge
+    int* scales;     // LDS, kRing/kPF entries: the producer's scale exponent C during the block that
+                     // produced entries [16b, 16b+16)  (linear walk only)
     int* produced;   // LDS, steps the producer has completed (INT_MAX when it is done)
     int* consumed;   // LDS, steps the consumer has completed
 };
@@ -318,7 +319,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     const int vo_sc = lane < nl ? lane * 4 : kOob;
     constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 64 wide
     constexpr int out_lane = BETA ? 0 : 63;
-    double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
+    double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
 
     clear_around<BETA>(r_cell, T, nl, lane);
@@ -358,17 +359,22 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         // The two counters and (speculatively) the incoming entries in ONE LDS round trip: LDS
         // serves a wave's requests in order, so entries read after a counter that already shows them
         // produced are the produced ones.  Only a counter that falls short sends the wave polling.
-        double2 en_first = make_double2(0.0, 0.0);
+        double en_first = 0.0;
+        int cp_first = 0;
         {
             int prod = 0x7fffffff, cons = 0x7fffffff;
             if (HAS_IN) prod = __hip_atomic_load(rin.produced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (HAS_OUT) cons = __hip_atomic_load(rout.consumed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             keep_order();
-            if (HAS_IN) en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+            if (HAS_IN) {
+                en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+                cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
+            }
             if (HAS_IN && prod < k0 + kPF + in_shift) {
                 wait_at_least(rin.produced, k0 + kPF + in_shift, status);
                 keep_order();
                 en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
+                cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
             }
             if (HAS_OUT && cons < k0 + kPF - kRing - out_shift) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
         }
@@ -382,15 +388,14 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
-            const double2 en = en_first;
-            double ev = en.x;
+            double ev = en_first;
             if (BETA) {
                 ev *= (double)edge;
                 edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p16 + 63 * 16 + 4, 0);
             }
             // entry k0+j feeds frame k0+j of the edge column: beyond the last frame it is junk
             const bool ok = k0 + jl < T && ev != 0.0;
-            cp = (int)en.y;
+            cp = cp_first;
             e_lane = ok ? ev : 0.0;
             // the largest of the kPF entries (they sit in every row of 16 lanes), for the edge lane
             int te = ok ? __builtin_amdgcn_frexp_exp(ev) - cp : kNoExp;
@@ -438,7 +443,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         if (lane >= nl) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
         if (HAS_IN) e_lane = __builtin_ldexp(e_lane, __builtin_amdgcn_readlane(C, in_lane) - cp);
         buf_store_i32(r_sc, vo_sc, __builtin_amdgcn_readfirstlane(blk * p4), C);  // wave-uniform, and said so
-        const double Cd = (double)__builtin_amdgcn_readlane(C, out_lane);
+        if (HAS_OUT) rout.scales[(k0 / kPF) & (kRing / kPF - 1)] = __builtin_amdgcn_readlane(C, out_lane);
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
             const float2 cn = buf_load_f2(r_cell, vo_p, (mi + dq * kPF) * p16);
@@ -454,7 +459,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
                 hi_seen = max(hi_seen, h);
             }
             buf_store_d(r_out, vo, qi * p8, a);
-            if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = make_double2(BETA ? a : pass, Cd);
+            if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = BETA ? a : pass;
             const float2 nx = ring[(j + 1) % kPF];
             mul_own = (double)nx.x;
             mul_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.y) : nx.y);
@@ -495,7 +500,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     const int vo = lane < nl ? lane * 8 : kOob;
     constexpr int out_lane = BETA ? 0 : 63;
     const int vo_bo = lane == out_lane ? 0 : kOob;
-    double2* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
+    double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
 
     clear_leading<BETA>(r_cell, T, nl, lane);
@@ -536,7 +541,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
         if (HAS_IN) {
             double ev;
             if (CONC) {
-                ev = rin.slots[(k0 + jl + in_shift) & (kRing - 1)].x;
+                ev = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
             } else {
                 ev = e_next;
                 e_next = buf_load_d(r_in, jl * 8, (k0 + kPF + in_shift) * 8);
@@ -564,7 +569,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
             buf_store_d(r_out, vo, qi * p8, a);
             if (HAS_OUT) {
                 const double h = BETA ? a : pass;  // alpha hands on a + L(t,u); beta plain a
-                if (CONC) ring_out[(k0 + j) & (kRing - 1)] = make_double2(h, 0.0);
+                if (CONC) ring_out[(k0 + j) & (kRing - 1)] = h;
                 else buf_store_d(r_bo, vo_bo, (k0 + j) * 8, h);
             }
             const float2 nx = ring[(j + 1) % kPF];
@@ -615,7 +620,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
     const i64* __restrict__ bnd_off, int* seqmode, const LpCell* lp, double* alpha,
     double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int* status) {
-    __shared__ double2 s_ring[kMaxWaves - 1][2 * kRing + 64];
+    __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
+    __shared__ int s_scale[kMaxWaves - 1][kRing / kPF];
     __shared__ int s_produced[kMaxWaves];
     __shared__ int s_consumed[kMaxWaves];
     __shared__ volatile int s_unsafe;
@@ -640,7 +646,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     int* scale = dir ? scale_b : scale_a;
     const int nl_last = Up - ((S - 1) << 6);
     Ring none;
-    none.slots = nullptr; none.produced = nullptr; none.consumed = nullptr;
+    none.slots = nullptr; none.scales = nullptr; none.produced = nullptr; none.consumed = nullptr;
 
     const bool concurrent = S <= W;
     const bool linear = concurrent && (seqmode[n] & 1) == 0;  // the gather pass's verdict on the log-probs
@@ -653,8 +659,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         const i64 base = pad + (i64)s * full_strip;
         const bool has_in = p > 0, has_out = p < S - 1;
         Ring rin = none, rout = none;
-        if (has_in) { rin.slots = s_ring[p - 1]; rin.produced = &s_produced[p - 1]; rin.consumed = &s_consumed[p - 1]; }
-        if (has_out) { rout.slots = s_ring[p]; rout.produced = &s_produced[p]; rout.consumed = &s_consumed[p]; }
+        if (has_in) { rin.slots = s_ring[p - 1]; rin.scales = s_scale[p - 1]; rin.produced = &s_produced[p - 1]; rin.consumed = &s_consumed[p - 1]; }
+        if (has_out) { rout.slots = s_ring[p]; rout.scales = s_scale[p]; rout.produced = &s_produced[p]; rout.consumed = &s_consumed[p]; }
         // alpha: the feeding strip's edge lane 63 trails its first lane by 63 steps; beta: the
         // feeding strip is s+1 and its edge lane 0 trails by its width - 1; likewise for the strip fed
         const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
