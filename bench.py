@@ -141,9 +141,22 @@ def main():
         loss.backward()
         return loss
 
+    # After any idle period (0.2 s is enough) this GPU runs the first ~12 ms of streaming work up to
+    # 15 % slower, whatever the kernels are.  Two priming steps let the allocator fetch its blocks
+    # (the device idles meanwhile), then ~25 ms of plain device copies, queued without a gap in
+    # front of the warm-up steps, bring the GPU to its steady state, so that a short --warmup does
+    # not measure that transient.
+    src = torch.empty(1 << 27, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    for _ in range(120):
+        dst.copy_(src)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    del src, dst
     # events between the steps (recorded, never waited on inside the timed region) give the spread
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
