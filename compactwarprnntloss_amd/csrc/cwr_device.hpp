@@ -245,6 +245,13 @@ __device__ __forceinline__ RowInfo decode_row(i64 r, i64 R, const i64* __restric
     return place_row(r, lo, R, row_off, lx, ly);
 }
 
+// Sets a bit of the status word.  A problem in the data usually shows in many rows at once: looking
+// first keeps them from queueing on one address (a batch whose labels all lie outside the
+// vocabulary took 2.5 ms instead of 0.2 in the gather pass).
+__device__ __forceinline__ void raise_flag(int* status, int bit) {
+    if ((__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0) atomicOr(status, bit);
+}
+
 __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restrict__ y, i64 y_stride,
                                            i64 y_len, const i64* __restrict__ lab_off, int V,
                                            int* status) {
@@ -252,7 +259,7 @@ __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restr
     i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : lab_off[ri.n]) + ri.u;
     int lab = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
     if (lab < 0 || lab >= V) {
-        if (status) atomicOr(status, CWR_FLAG_BAD_LABEL);
+        if (status) raise_flag(status, CWR_FLAG_BAD_LABEL);
         return -1;
     }
     return lab;

@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* 
         }
         if (ri.n < 0) continue;
         if (ri.t >= T_pad || ri.u >= Up_pad) {  // this cell lies outside the padded inputs
-            if (status && lane == 0) atomicOr(status, CWR_FLAG_BAD_LENGTH);
+            if (status && lane == 0) raise_flag(status, CWR_FLAG_BAD_LENGTH);
             continue;
         }
         fo[k] = ((i64)ri.n * T_pad + ri.t) * H;

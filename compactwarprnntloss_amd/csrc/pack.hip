@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void k_pack_rows(const U* __restrict__ src, U*
         }
         if (ri.n < 0) continue;
         if (ri.t >= T_pad || ri.u >= Up_pad) {  // this cell lies outside the padded array
-            if (status && lane == 0) atomicOr(status, CWR_FLAG_BAD_LENGTH);
+            if (status && lane == 0) raise_flag(status, CWR_FLAG_BAD_LENGTH);
             continue;
         }
         const U* ps = src + (((i64)ri.n * T_pad + ri.t) * Up_pad + ri.u) * units_per_row;

@@ -428,7 +428,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         if (ri.u < ri.U) {
             const i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : labbase) + ri.u;
             const int l = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
-            if (l < 0 || l >= V) atomicOr(status, CWR_FLAG_BAD_LABEL); else my_lab = l;
+            if (l < 0 || l >= V) raise_flag(status, CWR_FLAG_BAD_LABEL); else my_lab = l;
         }
         my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
     }
