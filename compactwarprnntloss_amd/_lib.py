@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("CWARP_RNNT_LIB") or os.path.join(HERE, "libcwarp_rnnt
 # enum cwr_dtype / cwr_mode / cwr_flag
 F32, F16, BF16, F64 = 0, 1, 2, 3
 MODE_LOGPROB, MODE_FUSED = 0, 1
+NOALLOC_SCRATCH_BYTES = 96 << 20  # CWR_NOALLOC_SCRATCH_BYTES
 FLAG_ROWS_MISMATCH, FLAG_BAD_LENGTH, FLAG_BAD_LABEL, FLAG_FB_MISMATCH, FLAG_U_TOO_LARGE, FLAG_INTERNAL = \
     1, 2, 4, 8, 16, 32
 FLAG_NAMES = {
@@ -37,6 +38,8 @@ SIGNATURES = {
     "cwr_offsets": (C.c_int, [_p, _p, _i64, _i64, _p, _p, _p, _p]),
     "cwr_forward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                               _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "cwr_forward_noalloc": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
+                                      _p, _p, _p, _p, _p, _p, _p, _p]),
     "cwr_loss": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                            _p, _sz, _p, _p, _p, _p, _p]),
     "cwr_forward_reduced": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,

@@ -1,10 +1,37 @@
 // extern "C" entry points of libcwarp_rnnt_hip.so: argument validation (host only, before any HIP
 // call), workspace carving and kernel sequencing.  Mirrors the orchestration of
 // cwarp_cuda.cpp:58-136 without its host synchronisations and allocations.
+#include <mutex>
+
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
+// Scratch of cwr_forward_noalloc: one copy per GPU, held from the moment the library's code is
+// loaded on that GPU until the process ends.  Host code never uses this name as an address (it is
+// a host-side stand-in); it asks the runtime for the device address once per GPU, below.
+static __device__ __align__(256) unsigned char scratch[CWR_NOALLOC_SCRATCH_BYTES];
+
 namespace cwr {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once known
+
+// Address of the current GPU's copy of `scratch`.  The first call on a GPU asks the runtime; later
+// calls are a table look-up.
+static int scratch_of_current_device(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return CWR_ERR_RUNTIME;
+    if (dev < 0 || dev >= kMaxDevices) return CWR_ERR_TOO_LARGE;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return CWR_ERR_RUNTIME;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return CWR_OK;
+}
 
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
@@ -145,7 +172,8 @@ const char* cwr_strerror(int status) {
         case CWR_ERR_BLANK: return "blank index outside [0, V)";
         case CWR_ERR_ALIGN: return "a buffer is not aligned to its element size";
         case CWR_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
-        case CWR_ERR_TOO_LARGE: return "a size exceeds what the kernels can index";
+        case CWR_ERR_TOO_LARGE: return "a size exceeds what the kernels can index (or the built-in scratch can hold)";
+        case CWR_ERR_RUNTIME: return "a HIP runtime call failed";
     }
     return "unknown status";
 }
@@ -219,6 +247,23 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* l
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
                         workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream,
                         true);
+}
+
+int cwr_forward_noalloc(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                        const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
+                        int64_t max_u, int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
+                        float* lse, float* grads, float* costs, void* stream) {
+    // everything the host can judge first, so that a call that cannot run touches no GPU
+    int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+    if (rc != CWR_OK) return rc;
+    if (max_u < 0) return CWR_ERR_SHAPE;
+    const size_t need = workspace_bytes(N, R, max_u);
+    if (need > (size_t)CWR_NOALLOC_SCRATCH_BYTES) return CWR_ERR_TOO_LARGE;
+    void* ws = nullptr;
+    rc = scratch_of_current_device(&ws);
+    if (rc != CWR_OK) return rc;
+    return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, ws, need, row_off,
+                        lab_off, status, rowinfo, lse, grads, costs, nullptr, stream, true);
 }
 
 int cwr_forward_reduced(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,

@@ -57,7 +57,8 @@ enum cwr_status {
     CWR_ERR_BLANK = 5,     /* blank outside [0, V) (cwarp_rnnt/__init__.py:50) */
     CWR_ERR_ALIGN = 6,     /* a buffer is not aligned to its element size */
     CWR_ERR_LAUNCH = 7,    /* the HIP runtime refused a launch */
-    CWR_ERR_TOO_LARGE = 8  /* a size exceeds what the kernels index */
+    CWR_ERR_TOO_LARGE = 8, /* a size exceeds what the kernels index, or what the built-in scratch holds */
+    CWR_ERR_RUNTIME = 9    /* a HIP runtime call other than a launch failed */
 };
 
 /* bits of status[0], written by the kernels */
@@ -130,6 +131,29 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
                 void* workspace, size_t workspace_bytes,
                 int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
                 float* lse, float* grads, float* costs, void* stream);
+
+/* cwr_forward for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * forward allocates eight tensors per call, cwarp_cuda_rnnt_kernel.cu:399-404).  Same arguments,
+ * outputs and results as cwr_forward, without the workspace: the scratch is an array of
+ * CWR_NOALLOC_SCRATCH_BYTES inside the library's device code, one copy per GPU, there for as long as
+ * the process lives.  The call makes no allocation of any kind.
+ *   - cwr_workspace_bytes(N, R, max_u) must not exceed CWR_NOALLOC_SCRATCH_BYTES, else
+ *     CWR_ERR_TOO_LARGE.  96 MiB: the N=32, T~175, U~50 batch (R = 3.1e5) needs 30 MiB, the
+ *     long-form N=4, T~1250, U~300 batch (R = 1.5e6) 71 MiB.
+ *   - The first call on a GPU looks the array's address up (hipGetSymbolAddress); make it outside
+ *     a stream capture.
+ *   - Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams,
+ *     two threads) race.  Calls in stream order on one stream are safe; nothing from an earlier
+ *     call is relied on, the kernels initialise what they read.
+ *   - The array holds the lattice state of the LAST call on that GPU only; cwr_export_lattice does
+ *     not reach it. */
+#define CWR_NOALLOC_SCRATCH_BYTES (96u << 20)
+int cwr_forward_noalloc(const void* x, int dtype, int64_t R, int64_t V,
+                        const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                        int64_t N, int32_t blank, int mode, int64_t max_u,
+                        int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
+                        float* lse, float* grads, float* costs, void* stream);
 
 /* Loss only (no gradient state).  Replaces _cwarp_rnnt_loss (cwarp_cuda.cpp:58-82 ->
  * gather_cuda_forward + cwarp_cuda_cal_costs): beta recursion only, costs = -beta[0][0]. */
