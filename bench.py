@@ -39,13 +39,15 @@ WORKLOADS = {
 
 
 def measured_traffic(kernel: str, config: int):
-    """HBM bytes per launch of `kernel`, from the committed rocprofv3 counter summary, or None."""
-    path = os.path.join(ROOT, "profiles", f"traffic_c{config}.json.txt")
+    """(HBM bytes per launch of `kernel`, file it was read from) from the committed rocprofv3 counter
+    summary of this configuration, or (None, None)."""
+    rel = os.path.join("profiles", f"traffic_c{config}.json.txt")
     try:
-        with open(path) as f:
-            return json.load(f).get(kernel)
+        with open(os.path.join(ROOT, rel)) as f:
+            val = json.load(f).get(kernel)
+        return val, (rel if val is not None else None)
     except (OSError, ValueError):
-        return None
+        return None, None
 
 
 def cpu_baseline(cfg, x_cpu, budget_s, dev_out):
@@ -111,10 +113,10 @@ def main():
         sys.exit("bench.py needs a GPU")
     import compactwarprnntloss_amd as pkg
     import cwarp_rnnt
-    from oracle import rnnt_oracle as orc
+    from compactwarprnntloss_amd import workloads
 
     dev = torch.device("cuda:0")
-    cfg = orc.make_config(args.config)
+    cfg = workloads.make_config(args.config)
     tdt = torch.float16 if cfg["dtype"] == "f16" else torch.float32
     g = torch.Generator(device="cpu").manual_seed(1000 + args.config)
     # generated on the host in fp32, rounded once to the storage type, then made resident
@@ -192,6 +194,7 @@ def main():
 
     grad_bytes = R * V * 2 * esize
     achieved = grad_bytes / (bwd_ms * 1e-3) / 1e9
+    traffic, traffic_source = measured_traffic("k_grad", args.config)
     result = {
         "metric": "fwd+bwd algorithmic HBM GB/s of the fused compact RNN-T loss (gather+loss+grad)",
         "value": round(bytes_step / (ms_step * 1e-3) / 1e9, 1),
@@ -214,7 +217,7 @@ def main():
                          "forward_nograd_call": round(nograd_ms, 4)},
         "roofline": {"bound": "hbm", "kernel": "k_grad (cwr_backward)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic("k_grad", args.config)},
+                     "traffic": traffic, "traffic_source": traffic_source},
     }
 
     if args.with_pack:

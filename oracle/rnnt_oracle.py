@@ -176,6 +176,17 @@ def log_softmax(x):
 # ---------------------------------------------------------------------------------------------
 # lattice (one sequence; lp has shape (T, U+1, 2): [...,0]=blank, [...,1]=label)
 # ---------------------------------------------------------------------------------------------
+def row_lse(xs, chunk=2048):
+    """float64 log-sum-exp of every row of xs (any float type), as max + log(sum(exp(x - max))).
+    Walks the rows in chunks so that the float64 temporaries stay small."""
+    out = np.empty(xs.shape[0])
+    for i in range(0, xs.shape[0], chunk):
+        c = np.asarray(xs[i : i + chunk], dtype=np.float64)
+        m = c.max(axis=-1)
+        out[i : i + chunk] = m + np.log(np.exp(c - m[:, None]).sum(axis=-1))
+    return out
+
+
 def _lse(a, b):
     """max + log1p(exp(-|a-b|)) (cwarp_cuda_rnnt_kernel.cu:22-29), float64, -inf safe."""
     a = np.asarray(a, dtype=np.float64)
@@ -291,18 +302,17 @@ def loss_and_grad(x, lx, y, ly, blank=0, mode="logprob", grad_out=None, want_den
         T, U = int(lx[n]), int(ly[n])
         Up = U + 1
         lab = np.asarray(labels_of(y, ly, n), dtype=np.int64)
-        xs = np.asarray(x[off[n] : off[n + 1]], dtype=np.float64)
+        xs = np.asarray(x[off[n] : off[n + 1]])  # storage type; widened to float64 where it is used
         if mode == "fused":
-            m = xs.max(axis=-1)
-            lse = m + np.log(np.exp(xs - m[:, None]).sum(axis=-1))
+            lse = row_lse(xs)
             lse_all[off[n] : off[n + 1]] = lse
         else:
             lse = np.zeros(xs.shape[0])
         u_of_row = np.arange(T * Up) % Up
         lp = np.zeros((T * Up, 2))
-        lp[:, 0] = xs[:, blank] - lse
+        lp[:, 0] = xs[:, blank].astype(np.float64) - lse
         ml = u_of_row < U
-        lp[ml, 1] = xs[ml, lab[u_of_row[ml]]] - lse[ml]
+        lp[ml, 1] = xs[ml, lab[u_of_row[ml]]].astype(np.float64) - lse[ml]
         gathered[off[n] : off[n + 1]] = lp
         lp3 = lp.reshape(T, Up, 2)
         a = alphas(lp3)
@@ -319,7 +329,7 @@ def loss_and_grad(x, lx, y, ly, blank=0, mode="logprob", grad_out=None, want_den
             rows = np.arange(T * Up)
             if mode == "fused":
                 gamma = -(G[:, 0] + G[:, 1])
-                g[:] = np.exp(xs - lse[:, None]) * gamma[:, None]
+                g[:] = np.exp(xs.astype(np.float64) - lse[:, None]) * gamma[:, None]
                 g[rows, blank] += G[:, 0]
                 np.add.at(g, (rows[ml], lab[u_of_row[ml]]), G[ml, 1])
             else:
@@ -408,67 +418,3 @@ def uniform_cost(T, U, V):
     """Closed form when every log-prob equals -log V:
     (T+U) log V - log C(T+U-1, U)."""
     return (T + U) * math.log(V) - math.log(math.comb(T + U - 1, U))
-
-
-# ---------------------------------------------------------------------------------------------
-# synthetic batches (the five benchmark configurations)
-# ---------------------------------------------------------------------------------------------
-def make_config(idx, seed=None, scale=1.0):
-    """Seeded synthetic batch for configuration idx in 1..5.
-
-    Returns dict(N, V, lx, ly (int32), y_padded (N,Umax) int32, y_cat (sum U,) int32, sigma,
-    dtype ('f32'|'f16'), R).  Logits are NOT generated here (they are large); use
-    make_logits().  `scale` < 1 shrinks the T/U ranges for quick tests.
-    """
-    rng = np.random.default_rng(idx if seed is None else seed)
-
-    def s(v, lo=1):
-        return max(lo, int(round(v * scale)))
-
-    if idx == 1:
-        N, V, sigma, dt = 4, 32, 1.0, "f32"
-        lx = rng.integers(8, 33, N)
-        ly = rng.integers(2, 11, N)
-    elif idx == 2:
-        N, V, sigma, dt = 32, 1024, 2.0, "f32"
-        lx = rng.integers(s(100), s(250) + 1, N)
-        ly = rng.integers(s(20), s(80) + 1, N)
-    elif idx == 3:
-        N, V, sigma, dt = 16, 4096, 1.0, "f16"
-        lx = rng.integers(s(150), s(300) + 1, N)
-        ly = rng.integers(s(40), s(120) + 1, N)
-    elif idx == 4:
-        N, V, sigma, dt = 64, 512, 1.0, "f32"
-        lx = np.clip(np.round(rng.lognormal(math.log(120 * scale), 0.6, N)), 1, s(600)).astype(np.int64)
-        ly = np.clip(np.round(rng.lognormal(math.log(max(30 * scale, 1.0)), 0.7, N)), 0, lx).astype(np.int64)
-        ly[3] = 0          # forced: a sequence with no labels
-        lx[7] = 1          # forced: a single-frame sequence
-        ly[7] = min(ly[7], 1)
-    elif idx == 5:
-        N, V, sigma, dt = 4, 128, 1.5, "f32"
-        lx = rng.integers(s(1000), s(1500) + 1, N)
-        ly = rng.integers(s(200), s(400) + 1, N)
-    else:
-        raise ValueError(idx)
-    lx = lx.astype(np.int32)
-    ly = ly.astype(np.int32)
-    Umax = int(ly.max())
-    yp = np.zeros((N, max(Umax, 1)), dtype=np.int32)
-    cat = []
-    for n in range(N):
-        lab = rng.integers(1, V, int(ly[n])).astype(np.int32)
-        yp[n, : ly[n]] = lab
-        cat.append(lab)
-    yc = np.concatenate(cat) if cat else np.zeros(0, dtype=np.int32)
-    yp = yp[:, :Umax] if Umax > 0 else yp[:, :0]
-    R = int(row_offsets_i64(lx, ly)[-1])
-    return dict(N=N, V=V, lx=lx, ly=ly, y_padded=yp, y_cat=yc, sigma=sigma, dtype=dt, R=R, idx=idx)
-
-
-def make_logits(cfg, seed=None):
-    """float32 (or float16 for config 3) compact logits N(0, sigma) of shape (R, V)."""
-    rng = np.random.default_rng(1000 + cfg["idx"] if seed is None else seed)
-    x = rng.standard_normal((cfg["R"], cfg["V"]), dtype=np.float32) * np.float32(cfg["sigma"])
-    if cfg["dtype"] == "f16":
-        x = x.astype(np.float16)
-    return x

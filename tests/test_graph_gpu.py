@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from compactwarprnntloss_amd import workloads as wl
 from oracle import rnnt_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -16,7 +17,7 @@ DEV = "cuda:0"
 @pytest.mark.parametrize("fused", [True, False])
 def test_graph_replays_match_eager(fused):
     import compactwarprnntloss_amd as pkg
-    cfg = orc.make_config(2, scale=0.2)
+    cfg = wl.make_config(2, scale=0.2)
     lx_np, ly_np = cfg["lx"].astype(np.int32), cfg["ly"].astype(np.int32)
     N, V, R = cfg["N"], 256, cfg["R"]
     gen = torch.Generator(device=DEV).manual_seed(1)

@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 import torch
 
+from compactwarprnntloss_amd import workloads as wl
 from oracle import rnnt_oracle as orc
 from test_parity_gpu import TORCH_DT
 
@@ -117,7 +118,7 @@ def test_join_full_size_properties():
     """Benchmark-sized call (N=32, T~U[100,250], U~U[20,80], H=512): the compact rows equal the
     broadcast sum at sampled cells, and with unit dh the backward returns the cell counts."""
     pkg = _pkg()
-    cfg = orc.make_config(2)
+    cfg = wl.make_config(2)
     lx, ly = cfg["lx"].astype(np.int32), cfg["ly"].astype(np.int32)
     N, H = len(lx), 512
     f = torch.randn(N, int(lx.max()), H, device=DEV).requires_grad_(True)

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 import torch
 
+from compactwarprnntloss_amd import workloads as wl
 from oracle import rnnt_oracle as orc
 
 
@@ -287,17 +288,17 @@ def test_label_equal_to_blank_follows_reference_overwrite_in_logprob_mode():
 
 def test_configs_are_seeded_and_in_range():
     for idx in range(1, 6):
-        c1 = orc.make_config(idx, scale=0.2 if idx != 1 else 1.0)
-        c2 = orc.make_config(idx, scale=0.2 if idx != 1 else 1.0)
+        c1 = wl.make_config(idx, scale=0.2 if idx != 1 else 1.0)
+        c2 = wl.make_config(idx, scale=0.2 if idx != 1 else 1.0)
         assert np.array_equal(c1["lx"], c2["lx"]) and np.array_equal(c1["y_cat"], c2["y_cat"])
         assert c1["lx"].dtype == np.int32 and c1["ly"].dtype == np.int32
         assert c1["lx"].min() >= 1 and c1["ly"].min() >= 0
         if len(c1["y_cat"]):
             assert c1["y_cat"].min() >= 1 and c1["y_cat"].max() < c1["V"]
         assert c1["R"] == int((c1["lx"].astype(np.int64) * (c1["ly"] + 1)).sum())
-    c4 = orc.make_config(4)
+    c4 = wl.make_config(4)
     assert c4["ly"].min() == 0 and c4["lx"].min() == 1 and c4["N"] == 64
-    c2 = orc.make_config(2)
+    c2 = wl.make_config(2)
     assert c2["N"] == 32 and c2["V"] == 1024 and 100 <= c2["lx"].min() and c2["lx"].max() <= 250
 
 
@@ -333,3 +334,12 @@ def test_join_rows_backward_matches_finite_differences(act):
             num[idx] = ((fn(p, g) - fn(m, g)) if which == 0 else (fn(f, p) - fn(f, m))) / (2 * eps)
         np.testing.assert_allclose(grad, num, atol=1e-7)
     assert np.all(df[0, 2:] == 0) and np.all(dg[0, 2:] == 0)   # padding gets no gradient
+
+
+def test_row_lse_matches_scipy_for_every_storage_type():
+    from scipy.special import logsumexp
+    rng = np.random.default_rng(3)
+    for dt in (np.float16, np.float32, np.float64):
+        x = (rng.standard_normal((5000, 37)) * 6).astype(dt)
+        x[17] = 30000 if dt == np.float16 else 1e4   # exp would overflow without the row maximum
+        np.testing.assert_allclose(orc.row_lse(x, chunk=999), logsumexp(x.astype(np.float64), axis=-1), rtol=1e-14)
