@@ -35,6 +35,8 @@ SIGNATURES = {
     "cwr_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "cwr_workspace_section": (C.c_int, [_i64, _i64, _i64, C.c_int, C.POINTER(_sz), C.POINTER(_sz)]),
     "cwr_lattice_slot": (_i64, [_i64, _i64, _i64, _i64]),
+    "cwr_cost_rule": (C.c_int, [C.c_double, C.c_double, C.POINTER(C.c_float)]),
+    "cwr_debug_wait_limit": (None, [C.c_int]),
     "cwr_offsets": (C.c_int, [_p, _p, _i64, _i64, _p, _p, _p, _p]),
     "cwr_forward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                               _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),

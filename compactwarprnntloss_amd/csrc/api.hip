@@ -1,6 +1,7 @@
 // extern "C" entry points of libcwarp_rnnt_hip.so: argument validation (host only, before any HIP
 // call), workspace carving and kernel sequencing.  Mirrors the orchestration of
 // cwarp_cuda.cpp:58-136 without its host synchronisations and allocations.
+#include <cstdio>
 #include <mutex>
 
 #include "cwr_device.hpp"
@@ -13,6 +14,8 @@ static __device__ __align__(256) unsigned char scratch[CWR_NOALLOC_SCRATCH_BYTES
 
 namespace cwr {
 
+thread_local int g_last_hip_error = 0;
+
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mu;
 static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once known
@@ -21,12 +24,14 @@ static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each
 // calls are a table look-up.
 static int scratch_of_current_device(void** out) {
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess) return CWR_ERR_RUNTIME;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return CWR_ERR_RUNTIME; }
     if (dev < 0 || dev >= kMaxDevices) return CWR_ERR_TOO_LARGE;
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     if (!g_scratch_ptr[dev]) {
         void* p = nullptr;
-        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return CWR_ERR_RUNTIME;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { g_last_hip_error = (int)e; return CWR_ERR_RUNTIME; }
         g_scratch_ptr[dev] = p;
     }
     *out = g_scratch_ptr[dev];
@@ -171,9 +176,16 @@ const char* cwr_strerror(int status) {
         case CWR_ERR_SHAPE: return "negative or inconsistent sizes";
         case CWR_ERR_BLANK: return "blank index outside [0, V)";
         case CWR_ERR_ALIGN: return "a buffer is not aligned to its element size";
-        case CWR_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
+        case CWR_ERR_LAUNCH:
+        case CWR_ERR_RUNTIME: {
+            // with the runtime's own words for the last failure seen by this thread
+            static thread_local char buf[192];
+            snprintf(buf, sizeof buf, "%s: %s", status == CWR_ERR_LAUNCH ? "the HIP runtime refused a kernel launch"
+                                                                         : "a HIP runtime call failed",
+                     hipGetErrorString((hipError_t)g_last_hip_error));
+            return buf;
+        }
         case CWR_ERR_TOO_LARGE: return "a size exceeds what the kernels can index (or the built-in scratch can hold)";
-        case CWR_ERR_RUNTIME: return "a HIP runtime call failed";
     }
     return "unknown status";
 }
@@ -186,6 +198,13 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u) {
 int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes) {
     return workspace_section(N, R, max_u, which, offset, bytes);
 }
+
+int cwr_cost_rule(double fwd_log2, double bwd_log2, float* cost) {
+    if (!cost) return -1;
+    return cost_rule(fwd_log2, bwd_log2, cost) ? 1 : 0;
+}
+
+void cwr_debug_wait_limit(int polls) { set_wait_limit(polls); }
 
 int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U) {
     if (t < 0 || u < 0 || t >= T || u > U) return -1;

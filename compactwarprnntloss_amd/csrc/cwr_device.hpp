@@ -198,6 +198,24 @@ struct __attribute__((aligned(16))) LpCell {
     float l_label;  // log2 P(y[u] | t,u); 0 in the last column
 };
 
+// Cost of a sequence from its two likelihoods, both as base-2 logarithms: fwd = alpha at the last
+// cell plus that cell's blank, bwd = beta[0][0].  cwarp_cuda_rnnt_kernel.cu:353-366: cost = -bwd,
+// unless the two differ by more than 0.1 % of the larger, in which case the reference prints a
+// warning and takes their mean; here the caller raises CWR_FLAG_FB_MISMATCH instead (returns true).
+// One deviation: the rule only fires when the two also differ by more than 1e-5 (in bits).  The
+// reference's rule is purely relative, and a likelihood within rounding of 1 (both logarithms of
+// the order of 1e-7) has no meaningful relative difference.
+__host__ __device__ inline bool cost_rule(double fwd_log2, double bwd_log2, float* cost) {
+    double fb = bwd_log2;
+    const double diff = fwd_log2 > fb ? fwd_log2 - fb : fb - fwd_log2;
+    const double larger = fwd_log2 > fb ? fwd_log2 : fb;
+    const double ratio = diff / (larger < 0 ? -larger : larger);
+    const bool mismatch = ratio > 1e-3 && diff > 1e-5;
+    if (mismatch) fb = (fwd_log2 + fb) * 0.5;
+    *cost = (float)(-fb * 0.6931471805599453);
+    return mismatch;
+}
+
 // Which sequence owns compact row r, and where in its lattice the row sits.
 struct RowInfo {
     int n;    // -1: the row belongs to no usable sequence
@@ -252,15 +270,23 @@ __device__ __forceinline__ void raise_flag(int* status, int bit) {
     if ((__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) == 0) atomicOr(status, bit);
 }
 
+// What a row's label slot can hold besides a label: nothing (the last column of a lattice emits no
+// label), or a label that does not exist (outside [0, V) or beyond the label array).  A bad label
+// poisons its sequence: the cost becomes NaN (bit kSeqPoisoned of the sequence's walk-mode word).
+constexpr int kNoLabel = -1;
+constexpr int kBadLabel = -2;
+constexpr int kSeqLogDomain = 1;  // walk-mode bits; 2 and 4 belong to the lattice kernel
+constexpr int kSeqPoisoned = 8;
+
 __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restrict__ y, i64 y_stride,
                                            i64 y_len, const i64* __restrict__ lab_off, int V,
                                            int* status) {
-    if (ri.n < 0 || ri.u >= ri.U) return -1;
+    if (ri.n < 0 || ri.u >= ri.U) return kNoLabel;
     i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : lab_off[ri.n]) + ri.u;
     int lab = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
     if (lab < 0 || lab >= V) {
         if (status) raise_flag(status, CWR_FLAG_BAD_LABEL);
-        return -1;
+        return kBadLabel;
     }
     return lab;
 }

@@ -87,8 +87,24 @@ int launch_join(int dtype, int act, bool backward, const void* a, const void* b,
                 const int* ly, const i64* row_off, i64 N, i64 T_pad, i64 Up_pad, i64 H, i64 R, int* status,
                 hipStream_t stream);
 
+// Launches go through CWR_LAUNCH, which first drops whatever error an earlier HIP call of this thread
+// (the caller's, or another library's) left pending, so that check_launch() reports this launch and
+// nothing else.  The runtime's own code is kept for cwr_strerror.
+#define CWR_LAUNCH(...)                      \
+    do {                                     \
+        (void)hipGetLastError();             \
+        hipLaunchKernelGGL(__VA_ARGS__);     \
+    } while (0)
+
+extern thread_local int g_last_hip_error;  // hipError_t of the last refused launch or failed call
+
 inline int check_launch() {
-    return hipGetLastError() == hipSuccess ? CWR_OK : CWR_ERR_LAUNCH;
+    const hipError_t e = hipGetLastError();
+    if (e == hipSuccess) return CWR_OK;
+    g_last_hip_error = (int)e;
+    return CWR_ERR_LAUNCH;
 }
+
+void set_wait_limit(int polls);  // lattice.hip: polls a wait inside k_lattice may spend (<= 0: default)
 
 }  // namespace cwr

@@ -113,9 +113,9 @@ __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* 
     RowInfo ri = decode_row(r0, R, row_off, lx, ly, N);
 #pragma unroll
     for (int k = 0; k < kJoinRows; ++k) {
-        fo[k] = -1; go[k] = -1;
+        fo[k] = -1; go[k] = -1;  // -1: a row of the output that no valid cell maps to (it is zeroed)
         const i64 r = r0 + k;
-        if (r >= R) continue;
+        if (r >= R) { fo[k] = -2; continue; }  // -2: beyond the output
         if (k > 0) {
             if (ri.n >= 0 && ri.u < ri.U) {
                 ++ri.u;
@@ -137,7 +137,14 @@ __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* 
     if (!FLAT) {  // rows of whole multiples of 64 packs: row after row, addresses on the scalar unit
 #pragma unroll
         for (int k = 0; k < kJoinRows; ++k) {
-            if (fo[k] < 0) continue;
+            if (fo[k] == -2) continue;
+            if (fo[k] < 0) {  // no uninitialised row ever reaches the output layer that follows
+                PackT<T, VEC> z;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) z.e[i] = Arith<T>::down(A(0));
+                for (int j = lane; j < NV; j += 64) st_stream<T, VEC>(out + (r0 + k) * H + j * VEC, z);
+                continue;
+            }
             const T* pf = f + fo[k];
             const T* pg = g + go[k];
             T* po = out + (r0 + k) * H;
@@ -167,8 +174,15 @@ __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* 
             a_at = past ? fo[q] : a_at;
             b_at = past ? go[q] : b_at;
         }
-        if (a_at < 0) continue;
+        if (a_at == -2) continue;
         const int col = (idx - k * NV) * VEC;
+        if (a_at < 0) {
+            PackT<T, VEC> z;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) z.e[i] = Arith<T>::down(A(0));
+            st_stream<T, VEC>(out + (r0 + k) * H + col, z);
+            continue;
+        }
         const PackT<T, VEC> a = ld<T, VEC>(f + a_at + col);
         const PackT<T, VEC> b = ld<T, VEC>(g + b_at + col);
         PackT<T, VEC> o;
@@ -274,11 +288,11 @@ static int join_launch(const JoinArgs& j, bool backward) {
         const i64 blocks = (j.R + 4 * kJoinRows - 1) / (4 * kJoinRows);
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
         if ((j.H / VEC) % 64 == 0)
-            hipLaunchKernelGGL((k_join<T, VEC, ACT, false>), dim3((unsigned)blocks), dim3(256), 0, j.stream,
+            CWR_LAUNCH((k_join<T, VEC, ACT, false>), dim3((unsigned)blocks), dim3(256), 0, j.stream,
                                static_cast<const T*>(j.a), static_cast<const T*>(j.b), j.lx, j.ly, j.row_off,
                                (int)j.N, (int)j.T_pad, (int)j.Up_pad, (int)j.H, j.R, static_cast<T*>(j.o1), j.status);
         else
-            hipLaunchKernelGGL((k_join<T, VEC, ACT, true>), dim3((unsigned)blocks), dim3(256), 0, j.stream,
+            CWR_LAUNCH((k_join<T, VEC, ACT, true>), dim3((unsigned)blocks), dim3(256), 0, j.stream,
                                static_cast<const T*>(j.a), static_cast<const T*>(j.b), j.lx, j.ly, j.row_off,
                                (int)j.N, (int)j.T_pad, (int)j.Up_pad, (int)j.H, j.R, static_cast<T*>(j.o1), j.status);
         return check_launch();
@@ -288,14 +302,14 @@ static int join_launch(const JoinArgs& j, bool backward) {
     for (i64 n0 = 0; n0 < j.N; n0 += 65535) {
         const unsigned nz = (unsigned)(j.N - n0 < 65535 ? j.N - n0 : 65535);
         if (j.T_pad > 0) {
-            hipLaunchKernelGGL((k_join_bwd_f<T, VEC, ACT>), dim3((unsigned)cblocks, (unsigned)j.T_pad, nz), dim3(256),
+            CWR_LAUNCH((k_join_bwd_f<T, VEC, ACT>), dim3((unsigned)cblocks, (unsigned)j.T_pad, nz), dim3(256),
                                0, j.stream, static_cast<const T*>(j.a), static_cast<const T*>(j.b), j.lx, j.ly,
                                j.row_off, (int)n0, (int)j.T_pad, (int)j.H, j.R, static_cast<T*>(j.o1));
             int rc = check_launch();
             if (rc != CWR_OK) return rc;
         }
         if (j.Up_pad > 0) {
-            hipLaunchKernelGGL((k_join_bwd_g<T, VEC, ACT>), dim3((unsigned)cblocks, (unsigned)j.Up_pad, nz), dim3(256),
+            CWR_LAUNCH((k_join_bwd_g<T, VEC, ACT>), dim3((unsigned)cblocks, (unsigned)j.Up_pad, nz), dim3(256),
                                0, j.stream, static_cast<const T*>(j.a), static_cast<const T*>(j.b), j.lx, j.ly,
                                j.row_off, (int)n0, (int)j.Up_pad, (int)j.H, j.R, static_cast<T*>(j.o2));
             int rc = check_launch();

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                    i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode,
                    int* status, float* costs, float* reduced, hipStream_t stream) {
-    hipLaunchKernelGGL(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
+    CWR_LAUNCH(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
                        row_off, lab_off, pad_off, slot_off, bnd_off, seqmode, status, costs, reduced);
     return check_launch();
 }
@@ -211,12 +211,24 @@ struct Ring {
     int* consumed;   // LDS, steps the consumer has completed
 };
 
-__device__ __forceinline__ bool wait_at_least(int* counter, int need, int* status) {
-    for (int spin = 0; spin < kSpinLimit; ++spin) {
+// What a wait needs besides its counter: where to report, the workgroup's abort word, and how many
+// polls to spend.  A wait that runs out sets the abort word; every later wait of the workgroup sees
+// it first and returns at once, so a broken hand-over costs ONE spin budget, not one per block.
+struct WaitCtl {
+    int* status;  // the call's status word (global)
+    int* abort;   // LDS, one per workgroup
+    int limit;    // polls
+};
+
+__device__ __forceinline__ bool wait_at_least(int* counter, int need, const WaitCtl& wc) {
+    if (__hip_atomic_load(wc.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0) return false;
+    for (int spin = 0; spin < wc.limit; ++spin) {
         if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= need) return true;
+        if (__hip_atomic_load(wc.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0) return false;
         __builtin_amdgcn_s_sleep(2);
     }
-    atomicOr(status, CWR_FLAG_INTERNAL);
+    __hip_atomic_store(wc.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    raise_flag(wc.status, CWR_FLAG_INTERNAL);
     return false;
 }
 
@@ -305,12 +317,13 @@ template <bool BETA, bool HAS_IN, bool HAS_OUT>
 __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const bool seed, const int in_shift,
                                                 const int out_shift, const LpCell* lp_strip,
                                                 double* out_strip, int* scale_strip, const Ring rin,
-                                                const Ring rout, int* status) {
+                                                const Ring rout, const WaitCtl wc) {
     const int lane = threadIdx.x & 63;
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
     const int p16 = nl * 16, p8 = nl * 8, p4 = nl * 4;
+    bool gave_up = false;
     const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * p4);
@@ -371,13 +384,15 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
                 cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
             }
             if (HAS_IN && prod < k0 + kPF + in_shift) {
-                wait_at_least(rin.produced, k0 + kPF + in_shift, status);
+                gave_up = !wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
                 keep_order();
                 en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
                 cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
             }
-            if (HAS_OUT && cons < k0 + kPF - kRing - out_shift) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+            if (HAS_OUT && cons < k0 + kPF - kRing - out_shift)
+                gave_up = !wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc) || gave_up;
         }
+        if ((HAS_IN || HAS_OUT) && gave_up) break;  // wave-uniform: the counters are
         keep_order();
         // Renew the scales.  True magnitude (binary exponent minus scale) of what the lane holds,
         // of what it will hand over and of what its neighbour will hand over next:
@@ -475,6 +490,10 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         if (HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    if (gave_up) {  // nobody is to wait for this strip any more
+        if (HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     return __ballot(lo_seen < kLowHigh - 1u || hi_seen >= kHighHigh) == 0;
 }
 
@@ -486,8 +505,9 @@ template <bool BETA, bool HAS_IN, bool HAS_OUT, bool CONC>
 __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const bool seed, const int in_shift,
                                                 const int out_shift, const LpCell* lp_strip,
                                                 double* out_strip, const double* bnd_in, double* bnd_out,
-                                                const Ring rin, const Ring rout, int* status) {
+                                                const Ring rin, const Ring rout, const WaitCtl wc) {
     const int lane = threadIdx.x & 63;
+    bool gave_up = false;
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
@@ -534,8 +554,9 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
         // entries [k0+in_shift, k0+kPF+in_shift) must have been produced; the ring slots of entries
         // [k0, k0+kPF) must be free, i.e. the consumer (which reads entry i at its step
         // i-out_shift) must be past entry k0+kPF-1-kRing
-        if (CONC && HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, status);
-        if (CONC && HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, status);
+        if (CONC && HAS_IN) gave_up = !wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
+        if (CONC && HAS_OUT) gave_up = !wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc) || gave_up;
+        if (CONC && gave_up) break;
         if (CONC) keep_order();
         double e_lane = kNeg;
         if (HAS_IN) {
@@ -585,12 +606,16 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
         if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    if (CONC && gave_up) {
+        if (HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
 }
 
 template <bool BETA>
 __device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
                                              int out_shift, const LpCell* lp, double* out, int* sc, Ring rin,
-                                             Ring rout, int* status) {
+                                             Ring rout, const WaitCtl status) {
     if (has_in && has_out) return sweep_strip_lin<BETA, true, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
     if (has_in) return sweep_strip_lin<BETA, true, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
     if (has_out) return sweep_strip_lin<BETA, false, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
@@ -600,7 +625,7 @@ __device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, i
 template <bool BETA, bool CONC>
 __device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
                                              int out_shift, const LpCell* lp, double* out, const double* bi,
-                                             double* bo, Ring rin, Ring rout, int* status) {
+                                             double* bo, Ring rin, Ring rout, const WaitCtl status) {
     if (has_in && has_out) sweep_strip_log<BETA, true, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
     else if (has_in) sweep_strip_log<BETA, true, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
     else if (has_out) sweep_strip_log<BETA, false, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
@@ -619,12 +644,14 @@ constexpr int kMaxWaves = 8;
 __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
     const i64* __restrict__ bnd_off, int* seqmode, const LpCell* lp, double* alpha,
-    double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int* status) {
+    double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int spin_limit,
+    int* status_word) {
     __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
     __shared__ int s_scale[kMaxWaves - 1][kRing / kPF];
     __shared__ int s_produced[kMaxWaves];
     __shared__ int s_consumed[kMaxWaves];
     __shared__ volatile int s_unsafe;
+    __shared__ int s_abort;
     const int n = blockIdx.x;
     const int dir = beta_only ? 1 : (int)blockIdx.y;
     const int W = blockDim.x >> 6;
@@ -634,8 +661,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         s_produced[threadIdx.x] = 0;
         s_consumed[threadIdx.x] = 0;
     }
-    if (threadIdx.x == 0) s_unsafe = 0;
+    if (threadIdx.x == 0) { s_unsafe = 0; s_abort = 0; }
     __syncthreads();
+    WaitCtl status;  // handed to every walk of this workgroup
+    status.status = status_word; status.abort = &s_abort; status.limit = spin_limit;
     const i64 pad = pad_off[n];
     if (pad < 0) return;
     const int T = lx[n], U = ly[n];
@@ -667,9 +696,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         const int out_shift = dir ? nl - 1 : 63;
         const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
         if (!linear) {
-            if (!active) return;
-            if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
-            else log_dispatch<true, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+            if (active) {
+                if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+                else log_dispatch<true, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+            }
+            __syncthreads();
+            // a hand-over that never came: the lattice is incomplete, the sequence's cost becomes NaN
+            if (s_abort != 0 && threadIdx.x == 0) raise_flag(&seqmode[n], kSeqPoisoned);
             return;
         }
         bool safe = true;
@@ -680,6 +713,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         }
         if (!safe && lane == 0) s_unsafe = 1;
         __syncthreads();
+        if (s_abort != 0) {
+            if (threadIdx.x == 0) raise_flag(&seqmode[n], kSeqPoisoned);
+            return;
+        }
         if (s_unsafe == 0 || w != 0) return;
         // Some strip of this direction left the range the linear walk is exact in: wave 0 walks
         // the whole direction again, strip by strip, in the log domain (below).
@@ -705,6 +742,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     }
 }
 
+// Polls a wait inside k_lattice may spend; settable from the host so that the give-up path can be
+// exercised (with a limit of 1 a strip that has to wait for its feeder gives up at once, and every
+// wave still leaves the kernel normally).
+static int g_wait_limit = kSpinLimit;
+void set_wait_limit(int polls) { g_wait_limit = polls > 0 ? polls : kSpinLimit; }
+static int wait_limit() { return g_wait_limit; }
+
 // one wave per strip of the longest label sequence the call admits, up to the concurrent limit
 static int lattice_waves(const Batch& b) {
     const i64 strips = (b.max_u + 64) / 64;
@@ -714,9 +758,9 @@ static int lattice_waves(const Batch& b) {
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
     if (b.N == 0) return CWR_OK;
     dim3 grid((unsigned)b.N, beta_only ? 1 : 2);
-    hipLaunchKernelGGL(k_lattice, grid, dim3(lattice_waves(b) * 64), 0, b.stream, b.lx, b.ly, ws.pad_off,
+    CWR_LAUNCH(k_lattice, grid, dim3(lattice_waves(b) * 64), 0, b.stream, b.lx, b.ly, ws.pad_off,
                        ws.bnd_off, ws.seqmode, ws.lp, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, ws.bnd_a,
-                       ws.bnd_b, beta_only ? 1 : 0, b.status);
+                       ws.bnd_b, beta_only ? 1 : 0, wait_limit(), b.status);
     return check_launch();
 }
 
@@ -882,17 +926,9 @@ __device__ __forceinline__ bool fill_slot(const int* __restrict__ lx, const int*
     }
     grads[r] = make_float2(gb, gl);
     if (t == T - 1 && u == U) {
-        // cwarp_cuda_rnnt_kernel.cu:353-366
-        double fa = a + (double)cell.l_blank;
-        double fb = b00;
-        double ratio = fabs(fa - fb) / fabs(fmax(fa, fb));
-        // the reference's rule is relative only; a likelihood within rounding of 1 (both logarithms
-        // ~1e-7) has no meaningful relative difference, hence the absolute floor
-        if (ratio > 1e-3 && fabs(fa - fb) > 1e-5) {
-            atomicOr(status, CWR_FLAG_FB_MISMATCH);
-            fb = (fa + fb) * 0.5;
-        }
-        costs[n] = (float)(-fb * (double)kLn2);
+        float cost;
+        if (cost_rule(a + (double)cell.l_blank, b00, &cost)) raise_flag(status, CWR_FLAG_FB_MISMATCH);
+        costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : cost;
         return true;
     }
     return false;
@@ -918,7 +954,7 @@ int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* 
     if (b.R == 0) return CWR_OK;
     const i64 slots = ws.slot_cap;  // the device knows the exact count; threads beyond it leave at once
     if ((slots + 255) / 256 > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(k_fill, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
+    CWR_LAUNCH(k_fill, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
                        ws.pad_off, ws.slot_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
                        ws.scale_b, reinterpret_cast<float2*>(grads), costs, reduced, b.status);
     (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
@@ -937,8 +973,9 @@ __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ l
     if (pad >= 0) {  // else: NaN already set by k_offsets
         LatticeView Bv;
         Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
-        Bv.linear = linear_beta(seqmode[n], (Bv.Up + 63) >> 6);
-        costs[n] = (float)(-Bv.log2_at(0, 0) * (double)kLn2);
+        const int mode = seqmode[n];
+        Bv.linear = linear_beta(mode, (Bv.Up + 63) >> 6);
+        costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : (float)(-Bv.log2_at(0, 0) * (double)kLn2);
         wrote = true;
     }
     finish_costs(wrote, N, costs, reduced, status);
@@ -946,7 +983,7 @@ __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ l
 
 int launch_cost_from_beta(const Batch& b, const Workspace& ws, float* costs, float* reduced) {
     if (b.N == 0) return CWR_OK;
-    hipLaunchKernelGGL(k_cost_from_beta, dim3((unsigned)((b.N + 63) / 64)), dim3(64), 0, b.stream, b.lx,
+    CWR_LAUNCH(k_cost_from_beta, dim3((unsigned)((b.N + 63) / 64)), dim3(64), 0, b.stream, b.lx,
                        b.ly, ws.pad_off, ws.seqmode, b.N, ws.beta, ws.scale_b, costs, reduced, b.status);
     return check_launch();
 }
@@ -988,7 +1025,7 @@ int launch_export(const int* lx, const int* ly, int N, i64 T_pad, i64 Up_pad, co
                   double* alphas_out, double* betas_out, hipStream_t stream) {
     const i64 total = (i64)N * T_pad * Up_pad;
     if (total == 0) return CWR_OK;
-    hipLaunchKernelGGL(k_export, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, lx, ly, ws.pad_off,
+    CWR_LAUNCH(k_export, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, lx, ly, ws.pad_off,
                        ws.seqmode, N, T_pad, Up_pad, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, alphas_out,
                        betas_out);
     return check_launch();

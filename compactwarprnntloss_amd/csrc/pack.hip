@@ -81,13 +81,17 @@ __global__ __launch_bounds__(256) void k_pack_rows(const U* __restrict__ src, U*
                 ri = decode_row(r, R, row_off, lx, ly, N);
             }
         }
-        if (ri.n < 0) continue;
-        if (ri.t >= T_pad || ri.u >= Up_pad) {  // this cell lies outside the padded array
+        U* pd = dst + r * units_per_row;
+        bool source = ri.n >= 0;
+        if (source && (ri.t >= T_pad || ri.u >= Up_pad)) {  // this cell lies outside the padded array
             if (status && lane == 0) raise_flag(status, CWR_FLAG_BAD_LENGTH);
+            source = false;
+        }
+        if (!source) {  // a row nothing maps to is zeroed: the loss never sees uninitialised memory
+            for (i64 j = lane; j < units_per_row; j += 64) Unit<U>::store(pd + j, Unit<U>::zero());
             continue;
         }
         const U* ps = src + (((i64)ri.n * T_pad + ri.t) * Up_pad + ri.u) * units_per_row;
-        U* pd = dst + r * units_per_row;
 #pragma unroll 4
         for (i64 j = lane; j < units_per_row; j += 64) Unit<U>::store(pd + j, Unit<U>::load(ps + j));
     }
@@ -103,7 +107,7 @@ static int repack_as(const void* src, void* dst, const int* lx, const int* ly, c
         const int rpw = row_bytes >= 4096 ? 1 : (int)(4096 / row_bytes < 8 ? 4096 / row_bytes : 8);
         const i64 blocks = (R + 4 * rpw - 1) / (4 * rpw);
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
-        hipLaunchKernelGGL((k_pack_rows<U>), dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<const U*>(src),
+        CWR_LAUNCH((k_pack_rows<U>), dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<const U*>(src),
                            static_cast<U*>(dst), lx, ly, row_off, (int)N, (int)T_pad, (int)Up_pad, units_per_row, R,
                            rpw, status);
         return check_launch();
@@ -113,7 +117,7 @@ static int repack_as(const void* src, void* dst, const int* lx, const int* ly, c
     for (i64 n0 = 0; n0 < N; n0 += 65535) {
         const i64 nz = N - n0 < 65535 ? N - n0 : 65535;
         dim3 grid((unsigned)(Up_pad * cblocks), (unsigned)T_pad, (unsigned)nz);
-        hipLaunchKernelGGL((k_unpack<U>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
+        CWR_LAUNCH((k_unpack<U>), grid, dim3(256), 0, stream, static_cast<const U*>(src),
                            static_cast<U*>(dst), lx, ly, row_off, (int)n0, (int)T_pad, (int)Up_pad,
                            units_per_row, (unsigned)cblocks, R);
         int rc = check_launch();

@@ -139,11 +139,15 @@ __device__ __forceinline__ float exp2_of_logprob(float b) {
     return b > -0.015625f ? series : fast_exp2(b);
 }
 
-__device__ __forceinline__ LpCell make_lp(float xb, float xl, const Lse lse, bool has_label, int* seqmode_n) {
+// lab: the row's label, kNoLabel or kBadLabel.  The walk-mode word is looked at before it is set: a
+// batch of steep logits marks its sequences from most rows at once, and unconditional atomics on one
+// address per sequence would queue.
+__device__ __forceinline__ LpCell make_lp(float xb, float xl, const Lse lse, int lab, int* seqmode_n) {
     const float b = (float)(((double)fmaxf(xb, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s);
-    const float l = has_label
+    const float l = lab >= 0
         ? (float)(((double)fmaxf(xl, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s) : 0.f;
-    if (!(b >= kLinMin && b <= kLinMax && l >= kLinMin && l <= kLinMax)) atomicOr(seqmode_n, 1);
+    if (!(b >= kLinMin && b <= kLinMax && l >= kLinMin && l <= kLinMax)) raise_flag(seqmode_n, kSeqLogDomain);
+    if (lab == kBadLabel) raise_flag(seqmode_n, kSeqPoisoned);
     LpCell c;
     c.p_blank = exp2_of_logprob(b);
     c.p_label = exp2_of_logprob(l);
@@ -314,8 +318,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     if (kFromRegs) { xb = rb; xl = rl; }
     if (lane == 0) {
         lse_out[r] = lse.value();
-        rowinfo[r] = make_int2(lab, ri.n);
-        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
+        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
     }
 }
@@ -428,7 +432,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         if (ri.u < ri.U) {
             const i64 at = (y_stride >= 0 ? (i64)ri.n * y_stride : labbase) + ri.u;
             const int l = (at >= 0 && at < y_len && (y_stride < 0 || ri.u < y_stride)) ? y[at] : -1;
-            if (l < 0 || l >= V) raise_flag(status, CWR_FLAG_BAD_LABEL); else my_lab = l;
+            if (l < 0 || l >= V) { raise_flag(status, CWR_FLAG_BAD_LABEL); my_lab = kBadLabel; } else my_lab = l;
         }
         my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
     }
@@ -461,8 +465,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     }
     if (mine) {
         lse_out[r] = res_lse.value();
-        rowinfo[r] = make_int2(my_lab, ri.n);
-        if (my_dst >= 0) lp[my_dst] = make_lp(res_b, res_l, res_lse, my_lab >= 0, seqmode + ri.n);
+        rowinfo[r] = make_int2(my_lab < 0 ? -1 : my_lab, ri.n);
+        if (my_dst >= 0) lp[my_dst] = make_lp(res_b, res_l, res_lse, my_lab, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
     }
 }
@@ -573,8 +577,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
     const Lse lse = {M, log2_of_sum(S)};
     if (lane == 0) {
         lse_out[r] = lse.value();
-        rowinfo[r] = make_int2(lab, ri.n);
-        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+        rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
+        if (dst >= 0) lp[dst] = make_lp(xb, xl, lse, lab, seqmode + ri.n);
         else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
     }
 }
@@ -621,11 +625,11 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_small(
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-            lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+            lp[dst] = make_lp(xb, xl, lse, lab, seqmode + ri.n);
         } else if (grads_skipped) {
             grads_skipped[r] = make_float2(0.f, 0.f);
         }
-        rowinfo[r] = make_int2(lab, ri.n);
+        rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
     }
 }
 
@@ -659,11 +663,11 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
             const i64 dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
             const float xb = Elem<T>::to_f32(row[blank]);
             const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-            lp[dst] = make_lp(xb, xl, lse, lab >= 0, seqmode + ri.n);
+            lp[dst] = make_lp(xb, xl, lse, lab, seqmode + ri.n);
         } else if (grads_skipped) {
             grads_skipped[r] = make_float2(0.f, 0.f);
         }
-        rowinfo[r] = make_int2(lab, ri.n);
+        rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
     }
 }
 
@@ -686,11 +690,11 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
         const T* row = x + r * (i64)V;
         const float xb = Elem<T>::to_f32(row[blank]);
         const float xl = lab >= 0 ? Elem<T>::to_f32(row[lab]) : 0.f;
-        lp[dst] = make_lp(xb, xl, Lse{0.f, 0.f}, lab >= 0, seqmode + ri.n);
+        lp[dst] = make_lp(xb, xl, Lse{0.f, 0.f}, lab, seqmode + ri.n);
     } else if (grads_skipped) {
         grads_skipped[r] = make_float2(0.f, 0.f);
     }
-    rowinfo[r] = make_int2(lab, ri.n);
+    rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -975,12 +979,12 @@ __global__ __launch_bounds__(256) void k_rowinfo(const int* __restrict__ lx, con
     if (r >= R) return;
     const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
     const int lab = ri.n >= 0 ? fetch_label(ri, y, y_stride, y_len, lab_off, V, nullptr) : -1;
-    rowinfo[r] = make_int2(lab, ri.n);
+    rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
 }
 
 int launch_rowinfo(const Batch& b, int* rowinfo) {
     if (b.R == 0) return CWR_OK;
-    hipLaunchKernelGGL(k_rowinfo, dim3((unsigned)((b.R + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly,
+    CWR_LAUNCH(k_rowinfo, dim3((unsigned)((b.R + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly,
                        b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, b.N, b.R, b.V,
                        reinterpret_cast<int2*>(rowinfo));
     return check_launch();
@@ -1038,7 +1042,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     if (b.R == 0) return CWR_OK;
     if (b.mode == CWR_MODE_LOGPROB) {
         unsigned blocks = (unsigned)((b.R + 255) / 256);
-        hipLaunchKernelGGL((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
+        CWR_LAUNCH((k_gather_logprob<T>), dim3(blocks), dim3(256), 0, b.stream, x, b.R, b.V, b.lx,
                            b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank,
                            ws.lp, ri, gz, ws.seqmode, b.status);
         return check_launch();
@@ -1050,14 +1054,14 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
         // grids are multiples of 8 workgroups, see logical_block
 #define CWR_ROW(KK)                                                                                  \
     if (lpr == 64 && k == KK) {                                                                      \
-        hipLaunchKernelGGL((k_gather_row<T, KK, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u), \
+        CWR_LAUNCH((k_gather_row<T, KK, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u), \
                            dim3(kWavesPerBlock * 64), 0, b.stream, CWR_ARGS);                        \
         return check_launch();                                                                       \
     }
 #define CWR_ROWS(L, KK, NP)                                                                          \
     if (lpr == L && k == KK) {                                                                       \
         const int rows = (64 / L) * NP;                                                              \
-        hipLaunchKernelGGL((k_gather_rows<T, L, KK, NP, kGatherNT>),                                 \
+        CWR_LAUNCH((k_gather_rows<T, L, KK, NP, kGatherNT>),                                 \
                            dim3((blocks_for_waves((b.R + rows - 1) / rows) + 7u) & ~7u),             \
                            dim3(kWavesPerBlock * 64), 0, b.stream, CWR_ARGS);                        \
         return check_launch();                                                                       \
@@ -1069,7 +1073,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
 #undef CWR_ARGS
     }
     if (base_aligned(b.x) && b.V >= 64 * Elem<T>::VEC) {  // long rows, or rows off the 16-byte grid
-        hipLaunchKernelGGL((k_gather_long<T, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u),
+        CWR_LAUNCH((k_gather_long<T, kGatherNT>), dim3((blocks_for_waves(b.R) + 7u) & ~7u),
                            dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride,
                            b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode,
                            b.status);
@@ -1078,7 +1082,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
     if (b.V < 64 * Elem<T>::VEC) {  // short rows off the packed paths
 #define CWR_SMALL(L, KM)                                                                             \
     if (b.V <= L * KM) {                                                                             \
-        hipLaunchKernelGGL((k_gather_small<T, L, KM>), dim3(blocks_for_waves((b.R + 64 / L - 1) / (64 / L))), \
+        CWR_LAUNCH((k_gather_small<T, L, KM>), dim3(blocks_for_waves((b.R + 64 / L - 1) / (64 / L))), \
                            dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, \
                            b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz,     \
                            ws.seqmode, b.status);                                                    \
@@ -1087,7 +1091,7 @@ static int gather_typed(const Batch& b, const Workspace& ws, float* lse, int* ro
         CWR_SMALL(8, 4) CWR_SMALL(8, 8) CWR_SMALL(16, 8) CWR_SMALL(32, 8) CWR_SMALL(64, 8)
 #undef CWR_SMALL
     }
-    hipLaunchKernelGGL((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
+    CWR_LAUNCH((k_gather_fused_generic<T>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64),
                        0, b.stream, x, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off,
                        ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);
     return check_launch();
@@ -1106,7 +1110,7 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
         const int NV = b.V / Elem<T>::VEC;
         if (NV % 64 == 0 && b.R * (i64)(NV / 64) < 0x7fffffffLL) {  // (2^31 chunks of 1 KiB would be 2 TiB)
             const int ch = NV / 64;
-            hipLaunchKernelGGL((k_grad_flat<T, FUSED, kGradNT>), dim3((blocks_for_waves(b.R * ch) + 7u) & ~7u),
+            CWR_LAUNCH((k_grad_flat<T, FUSED, kGradNT>), dim3((blocks_for_waves(b.R * ch) + 7u) & ~7u),
                                dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ch, ri, g2,
                                lse, grad_costs, gx);
             return check_launch();
@@ -1116,7 +1120,7 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
             unsigned blocks = blocks_for_waves((b.R + rp - 1) / rp);
 #define CWR_CASE(L, KK)                                                                              \
     if (lpr == L && k == KK) {                                                                       \
-        hipLaunchKernelGGL((k_grad<T, FUSED, L, KK, kGradNT>), dim3(blocks), dim3(kWavesPerBlock * 64), \
+        CWR_LAUNCH((k_grad<T, FUSED, L, KK, kGradNT>), dim3(blocks), dim3(kWavesPerBlock * 64), \
                            0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);     \
         return check_launch();                                                                       \
     }
@@ -1127,7 +1131,7 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
     if (base_aligned(grad_x) && (!FUSED || base_aligned(b.x)) && b.V >= 64 * Elem<T>::VEC) {
         const i64 per_wave = 64 * Elem<T>::VEC;
         const i64 waves = (b.R * (i64)b.V + per_wave - 1) / per_wave;
-        hipLaunchKernelGGL((k_grad_any<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
+        CWR_LAUNCH((k_grad_any<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
                            dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse,
                            grad_costs, gx);
         return check_launch();
@@ -1135,12 +1139,12 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
     if (base_aligned(grad_x) && (!FUSED || base_aligned(b.x)) && b.V >= Elem<T>::VEC) {
         const i64 per_wave = 64 * Elem<T>::VEC;
         const i64 waves = (b.R * (i64)b.V + per_wave - 1) / per_wave;
-        hipLaunchKernelGGL((k_grad_small<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
+        CWR_LAUNCH((k_grad_small<T, FUSED, kGradNT>), dim3((blocks_for_waves(waves) + 7u) & ~7u),
                            dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse,
                            grad_costs, gx);
         return check_launch();
     }
-    hipLaunchKernelGGL((k_grad_generic<T, FUSED>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64), 0,
+    CWR_LAUNCH((k_grad_generic<T, FUSED>), dim3(blocks_for_waves(b.R)), dim3(kWavesPerBlock * 64), 0,
                        b.stream, x, b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);
     return check_launch();
 }

@@ -11,18 +11,17 @@ from typing import Any, Optional
 import torch
 
 from . import _lib
-from .loss import _DTYPES, _offsets, _stream_ptr
+from .loss import _DTYPES, _offsets, _raise_on_status, _stream_ptr
 
 _ACTS = {None: 0, "none": 0, "tanh": 1, "relu": 2}
 
 
 class _Join(torch.autograd.Function):
     @staticmethod
-    def forward(ctx: Any, f, g, lx, ly, total_rows, act):
+    def forward(ctx: Any, f, g, lx, ly, total_rows, act, row_off, status):
         lib = _lib.load()
         N, T, H = f.shape
         Up = g.size(1)
-        row_off, status = _offsets(lx, ly, total_rows)
         out = torch.empty((total_rows, H), dtype=f.dtype, device=f.device)
         with torch.cuda.device(f.device):
             rc = lib.cwr_join(f.data_ptr(), g.data_ptr(), _DTYPES[f.dtype], act, N, T, Up, H, lx.data_ptr(),
@@ -32,7 +31,6 @@ class _Join(torch.autograd.Function):
         ctx.save_for_backward(lx, ly, row_off, out if act else None)
         ctx.dims = (N, T, Up, H)
         ctx.act = act
-        ctx.status = status
         return out
 
     @staticmethod
@@ -49,17 +47,20 @@ class _Join(torch.autograd.Function):
                                        row_off.data_ptr(), dh.size(0), df.data_ptr(), dg.data_ptr(),
                                        _stream_ptr(dh.device))
             _lib.check(rc, "cwr_join_backward")
-        return df, dg, None, None, None, None
+        return df, dg, None, None, None, None, None, None
 
 
 def compact_join(f: torch.Tensor, g: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
-                 activation: Optional[str] = None, total_rows: Optional[int] = None) -> torch.Tensor:
+                 activation: Optional[str] = None, total_rows: Optional[int] = None,
+                 validate: bool = False) -> torch.Tensor:
     """h[row(n,t,u), :] = act(f[n, t, :] + g[n, u, :]) for t < lx[n], u <= ly[n], as (R, H) compact
     rows (sequence-major, then t, then u).  Differentiable in f and g.
 
     f: (N, T, H) encoder frames; g: (N, U+1, H) predictor states; lx, ly: (N,) int32 frame and label
     counts; activation: None, "tanh" or "relu"; total_rows: sum_i lx_i*(ly_i+1) if known, else it is
-    computed on the device and read back (one synchronisation)."""
+    computed on the device and read back (one synchronisation); validate: read the status word
+    back (one synchronisation) and raise when the lengths do not add up to total_rows or a sequence
+    does not fit f / g.  Without it the rows no valid cell maps to are zeros."""
     if activation not in _ACTS:
         raise RuntimeError(f"activation must be one of {sorted(k for k in _ACTS if k)} or None")
     if f.dim() != 3 or g.dim() != 3 or f.size(0) != g.size(0) or f.size(2) != g.size(2):
@@ -75,7 +76,11 @@ def compact_join(f: torch.Tensor, g: torch.Tensor, lx: torch.Tensor, ly: torch.T
         raise RuntimeError("lx, ly must hold one entry per sequence")
     if total_rows is None:
         total_rows = int((lx.long() * (ly.long() + 1)).sum().item())
-    return _Join.apply(f.contiguous(), g.contiguous(), lx, ly, int(total_rows), _ACTS[activation])
+    row_off, status = _offsets(lx, ly, int(total_rows))
+    out = _Join.apply(f.contiguous(), g.contiguous(), lx, ly, int(total_rows), _ACTS[activation], row_off, status)
+    if validate:
+        _raise_on_status(status, "compact_join")
+    return out
 
 
 class CompactJoiner(torch.nn.Module):

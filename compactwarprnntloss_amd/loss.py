@@ -11,7 +11,9 @@ additive keyword arguments:
                      fused into the gather pass, the gradient w.r.t. the logits is dense.
   x of 4 dims        a padded (N, T, U+1, V) tensor is packed first (pack_padded), as the
                      reference does through gather.cat (cwarp_rnnt/__init__.py:52-59)
-  max_u              host-known upper bound of max(ly) for concatenated 1-D labels
+  max_u              host-known upper bound of max(ly).  Padded labels give one for free (their
+                     width); with concatenated 1-D labels and no max_u the maximum of ly is read
+                     back from the device (one synchronisation per call)
   validate           read the device status word back (one synchronisation) and raise on
                      data-dependent problems.  Off by default: the hot path never synchronises.
 """
@@ -73,7 +75,11 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     R, V = xs.shape
     y_stride, y_len = _label_args(ys)
     if max_u is None:
-        max_u = ys.size(1) if ys.dim() == 2 else ys.numel()
+        # padded labels bound max(ly) by their width.  Concatenated labels carry no such bound (their
+        # total would size the workspace and the lattice kernel for one sequence holding every label
+        # of the batch: 8x the memory on a typical batch), so the true maximum is read back: one
+        # synchronisation, which callers avoid by passing max_u.
+        max_u = ys.size(1) if ys.dim() == 2 else (int(ly.max().item()) if ly.numel() else 0)
     mode = _lib.MODE_FUSED if fused else _lib.MODE_LOGPROB
 
     st = ForwardState()
@@ -177,10 +183,9 @@ class _Pack(torch.autograd.Function):
     """Padded (N, T, U+1, V) -> compact (R, V) and its backward (cwr_pack / cwr_unpack)."""
 
     @staticmethod
-    def forward(ctx: Any, x4, lx, ly, total_rows):
+    def forward(ctx: Any, x4, lx, ly, total_rows, row_off, status):
         lib = _lib.load()
         N, T, Up, V = x4.shape
-        row_off, status = _offsets(lx, ly, total_rows)
         out = torch.empty((total_rows, V), dtype=x4.dtype, device=x4.device)
         with torch.cuda.device(x4.device):
             rc = lib.cwr_pack(x4.data_ptr(), _DTYPES[x4.dtype], N, T, Up, V, lx.data_ptr(), ly.data_ptr(),
@@ -189,7 +194,6 @@ class _Pack(torch.autograd.Function):
             _lib.check(rc, "cwr_pack")
         ctx.save_for_backward(lx, ly, row_off)
         ctx.shape = (N, T, Up, V)
-        ctx.status = status
         return out
 
     @staticmethod
@@ -203,11 +207,19 @@ class _Pack(torch.autograd.Function):
             rc = lib.cwr_unpack(g.data_ptr(), _DTYPES[g.dtype], N, T, Up, V, lx.data_ptr(), ly.data_ptr(),
                                 row_off.data_ptr(), g.size(0), out.data_ptr(), _stream_ptr(g.device))
             _lib.check(rc, "cwr_unpack")
-        return out, None, None, None
+        return out, None, None, None, None, None
+
+
+def _raise_on_status(status: torch.Tensor, what: str):
+    """Reads a status word back (one synchronisation) and raises on any problem but a
+    forward/backward mismatch, which the reference only reports."""
+    hard = int(status[0].item()) & ~_lib.FLAG_FB_MISMATCH
+    if hard:
+        raise RuntimeError(f"{what}: " + _lib.describe_flags(hard))
 
 
 def pack_padded(x: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
-                total_rows: Optional[int] = None) -> torch.Tensor:
+                total_rows: Optional[int] = None, validate: bool = False) -> torch.Tensor:
     """Compact layout (sum_i T_i*(U_i+1), V) of a padded joiner output (N, T, U+1, V): for every
     sequence the rows of its own T_i x (U_i+1) sub-lattice, t-major (test/test.py:44-46).
     Differentiable.  Takes the place of `gather.cat` in cwarp_rnnt/__init__.py:52-59, which keeps the
@@ -215,7 +227,11 @@ def pack_padded(x: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
     compact layout when every U_i equals the padded width.
 
     total_rows: sum_i T_i*(U_i+1) if the caller knows it; otherwise it is computed on the device and
-    read back (one synchronisation)."""
+    read back (one synchronisation).
+    validate: read the status word back (one synchronisation) and raise when the lengths do not add
+    up to total_rows or a sequence does not fit the padded tensor (the reference asserts
+    `lx.max() == T` and `y.size(1)+1 == Up`, cwarp_rnnt/__init__.py:57-58).  Without it such rows
+    are zeros, never uninitialised memory."""
     if x.dim() != 4:
         raise RuntimeError("x must be (N, T, U+1, V)")
     if not x.is_cuda or not x.is_contiguous():
@@ -229,14 +245,15 @@ def pack_padded(x: torch.Tensor, lx: torch.Tensor, ly: torch.Tensor,
         raise RuntimeError("lx, ly must hold one entry per sequence")
     if total_rows is None:
         total_rows = int((lx.long() * (ly.long() + 1)).sum().item())
-    return _Pack.apply(x, lx, ly, int(total_rows))
+    row_off, status = _offsets(lx, ly, int(total_rows))
+    out = _Pack.apply(x, lx, ly, int(total_rows), row_off, status)
+    if validate:
+        _raise_on_status(status, "pack_padded")
+    return out
 
 
 def _raise_on_flags(st: ForwardState):
-    flags = int(st.status[0].item())
-    hard = flags & ~_lib.FLAG_FB_MISMATCH
-    if hard:
-        raise RuntimeError("transducer_loss: " + _lib.describe_flags(hard))
+    _raise_on_status(st.status, "transducer_loss")
 
 
 class _TransLoss(torch.autograd.Function):
@@ -304,7 +321,10 @@ def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torc
         import warnings
         warnings.warn("transducer_loss: 4-D input is packed into the compact layout first; pass compact "
                       "(sum_i T_i*(U_i+1), V) input to skip that copy", stacklevel=2)
-        x = pack_padded(x if x.is_contiguous() else x.contiguous(), lx, ly)
+        if y.dim() == 2:
+            # cwarp_rnnt/__init__.py:57 asserts y.size(1)+1 == Up; a wider padded tensor is fine here
+            assert y.size(1) + 1 <= x.size(2), "x must hold U+1 label positions"
+        x = pack_padded(x if x.is_contiguous() else x.contiguous(), lx, ly, validate=bool(validate))
     # x: (STU, V)
     assert x.dim() == 2, "input must be compact: (sum_i T_i*(U_i+1), V)"
 
@@ -317,7 +337,7 @@ def transducer_loss(x: torch.Tensor, lx: torch.Tensor, y: torch.Tensor, ly: torc
 def rnnt_loss(log_probs: torch.Tensor, labels: torch.Tensor, frames_lengths: torch.Tensor,
               labels_lengths: torch.Tensor, average_frames: bool = False, reduction: Optional[str] = None,
               blank: int = 0, gather: bool = False, fastemit_lambda: float = 0.0,
-              compact: bool = False) -> torch.Tensor:
+              compact: bool = False, max_u: Optional[int] = None) -> torch.Tensor:
     """Front end with the call signature of `warp_rnnt.rnnt_loss`, the sibling API the reference's own
     test drives next to `transducer_loss` (test/test.py:4,67), on top of the same kernels.
 
@@ -328,6 +348,8 @@ def rnnt_loss(log_probs: torch.Tensor, labels: torch.Tensor, frames_lengths: tor
     gather          accepted; the gather of the blank and label columns is always on here
     fastemit_lambda scales the gradient of every label emission by (1 + lambda) and leaves the loss
                     value alone (FastEmit as a gradient re-weighting)
+    max_u           (not in warp_rnnt) upper bound of max(labels_lengths) known to the host; without
+                    it, concatenated labels cost one synchronisation per call to read the maximum back
     """
     assert reduction in (None, "none", "mean", "sum")
     del gather
@@ -342,7 +364,7 @@ def rnnt_loss(log_probs: torch.Tensor, labels: torch.Tensor, frames_lengths: tor
         x = pack_padded(x if x.is_contiguous() else x.contiguous(), lx, ly)
     elif x.dim() != 2:
         raise RuntimeError("compact log_probs must be (sum_i T_i*(U_i+1), V)")
-    costs = _TransLoss.apply(x, lx, labels.contiguous(), ly, int(blank), False, None, False, "none",
+    costs = _TransLoss.apply(x, lx, labels.contiguous(), ly, int(blank), False, max_u, False, "none",
                              float(fastemit_lambda))
     if average_frames:
         costs = costs / lx.to(costs.dtype)

@@ -65,13 +65,15 @@ enum cwr_status {
 enum cwr_flag {
     CWR_FLAG_ROWS_MISMATCH = 1, /* sum lx*(ly+1) != R */
     CWR_FLAG_BAD_LENGTH = 2,    /* some lx <= 0 or ly < 0 (that sequence is skipped, cost = NaN) */
-    CWR_FLAG_BAD_LABEL = 4,     /* a label outside [0, V) was met (treated as "no label") */
+    CWR_FLAG_BAD_LABEL = 4,     /* a label outside [0, V) or beyond the label array was met (that
+                                   sequence's cost is NaN) */
     CWR_FLAG_FB_MISMATCH = 8,   /* forward and backward log-likelihood differ by > 0.1 % (and by
                                    more than 1e-5, so that a likelihood within rounding of 1 does
                                    not count) for some sequence; the cost is their mean, as in the
                                    reference (cwarp_cuda_rnnt_kernel.cu:356-364, which prints) */
     CWR_FLAG_U_TOO_LARGE = 16,  /* some ly exceeds the max_u given to the call */
-    CWR_FLAG_INTERNAL = 32      /* a bounded wait inside a kernel ran out (results are invalid) */
+    CWR_FLAG_INTERNAL = 32      /* a bounded wait inside a kernel ran out (the cost of the sequence it
+                                   happened in is NaN) */
 };
 
 int cwr_version(void);
@@ -101,6 +103,21 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
  * C = scale[(pad_off[n] + s*(T+127)*64)/16 + (k/16)*nl + l].  cwr_export_lattice does this. */
 int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes);
 int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
+
+/* Host helper: the rule that turns a sequence's two likelihoods into its cost, exactly as the
+ * kernels apply it (cwarp_cuda_rnnt_kernel.cu:345-366).  fwd_log2 = log2 of alpha at the last cell
+ * times that cell's blank probability, bwd_log2 = log2 beta[0][0].  *cost = -bwd in nats; when the
+ * two differ by more than 0.1 % of the larger (and by more than 1e-5 bits: a floor the reference
+ * does not have, for likelihoods within rounding of 1) the cost is minus their mean and the
+ * function returns 1 -- the case in which the kernels raise CWR_FLAG_FB_MISMATCH and the reference
+ * prints a warning.  Returns 0 otherwise, -1 for a NULL cost. */
+int cwr_cost_rule(double fwd_log2, double bwd_log2, float* cost);
+
+/* Diagnostic: the number of polls a wave of the lattice kernel spends waiting for the neighbouring
+ * strip's wave before it gives up (CWR_FLAG_INTERNAL; the sequence's cost becomes NaN; every wave
+ * still leaves the kernel normally).  polls <= 0 restores the default (about 4 million).  Process-
+ * wide; meant for tests of that path. */
+void cwr_debug_wait_limit(int polls);
 
 /* Row and label offsets by a device prefix scan.
  *   row_off[n] = sum_{j<n} lx[j]*(ly[j]+1), n = 0..N   (N+1 entries, int64)
@@ -224,8 +241,9 @@ int cwr_export_lattice(const int32_t* lx, const int32_t* ly, int64_t N, int64_t 
  * u <= ly[n] (the compact order of test/test.py:44-46).
  *   x_padded (N, T_pad, Up_pad, V) contiguous;  x_compact (R, V);  row_off from cwr_offsets
  *   status   optional 4 x int32 already initialised by cwr_offsets: CWR_FLAG_BAD_LENGTH is added
- *            when a sequence does not fit (lx[n] > T_pad or ly[n]+1 > Up_pad); its rows beyond the
- *            padded array are left untouched. */
+ *            when a sequence does not fit (lx[n] > T_pad or ly[n]+1 > Up_pad).
+ * Every row of x_compact is written: rows whose cell lies beyond the padded array, and rows that
+ * belong to no sequence (R larger than the lengths add up to), are zeroed. */
 int cwr_pack(const void* x_padded, int dtype, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t V,
              const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* x_compact,
              int32_t* status, void* stream);
@@ -243,7 +261,7 @@ int cwr_unpack(const void* g_compact, int dtype, int64_t N, int64_t T_pad, int64
  * logits to cwarp_rnnt/__init__.py:52-59); the linear layer that follows is left to a library GEMM
  * over the (R, H) rows.
  *   f (N, T_pad, H), g (N, Up_pad, H) contiguous;  h (R, H);  act a cwr_activation
- *   status as for cwr_pack. */
+ *   status as for cwr_pack; rows of h no valid cell maps to are zeroed, as there. */
 enum cwr_activation { CWR_ACT_NONE = 0, CWR_ACT_TANH = 1, CWR_ACT_RELU = 2 };
 int cwr_join(const void* f, const void* g, int dtype, int act, int64_t N, int64_t T_pad, int64_t Up_pad, int64_t H,
              const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* h, int32_t* status,

@@ -218,3 +218,49 @@ def test_golden_fixtures_match_the_oracle():
         np.testing.assert_allclose(out["G"], z["G"], rtol=1e-10, atol=1e-14)
         np.testing.assert_allclose(out["grad"], z["grad"], rtol=1e-10, atol=1e-14)
         assert np.array_equal(orc.row_offsets(z["lx"], z["ly"]), z["row_off_i32"])
+
+
+def test_cost_rule_matches_the_oracle_including_the_averaging_branch():
+    """cwarp_cuda_rnnt_kernel.cu:345-366 as the kernels apply it (the same host/device function),
+    against the oracle's cost_with_check: agreement, the 0.1 % mismatch with its averaging, and the
+    one documented deviation (no mismatch below 1e-5 bits of difference)."""
+    import ctypes as C
+    import math
+    import numpy as np
+    from oracle import rnnt_oracle as orc
+    lib = _lib.load()
+    ln2 = math.log(2.0)
+
+    def oracle(fa, fb):  # a 1 x 1 lattice whose forward / backward log-likelihoods are fa / fb (nats)
+        lp = np.zeros((1, 1, 2))
+        lp[0, 0, 0] = -1.0
+        return orc.cost_with_check(lp, np.array([[fa + 1.0]]), np.array([[fb]]))
+
+    def device_rule(fa, fb):
+        cost = C.c_float()
+        rc = lib.cwr_cost_rule(fa / ln2, fb / ln2, C.byref(cost))
+        return cost.value, rc
+
+    rng = np.random.default_rng(0)
+    seen = {0: 0, 1: 0}
+    for _ in range(2000):
+        fb = -float(rng.uniform(1e-3, 900.0))
+        rel = float(rng.choice([0.0, 1e-6, 5e-4, 9.9e-4, 1.01e-3, 2e-3, 5e-2])) * float(rng.choice([-1, 1]))
+        fa = fb * (1.0 + rel)
+        want, want_mis = oracle(fa, fb)
+        got, rc = device_rule(fa, fb)
+        assert rc == int(want_mis), (fa, fb, rel)
+        assert abs(got - want) <= 1e-6 * abs(want)
+        seen[rc] += 1
+    assert seen[0] > 200 and seen[1] > 200
+    # the averaging itself, on numbers one can do in one's head
+    got, rc = device_rule(-10.0, -12.0)
+    assert rc == 1 and abs(got - 11.0) < 1e-6
+    got, rc = device_rule(-12.0, -12.0)
+    assert rc == 0 and abs(got - 12.0) < 1e-6
+    # deviation: likelihoods within rounding of 1.  Relative difference 50 %, absolute 1e-7 nats:
+    # the reference's rule fires, this one does not and keeps -beta[0][0]
+    want, want_mis = oracle(-2e-7, -1e-7)
+    got, rc = device_rule(-2e-7, -1e-7)
+    assert want_mis and rc == 0 and abs(got - 1e-7) < 1e-12
+    assert lib.cwr_cost_rule(0.0, 0.0, None) == -1

@@ -240,8 +240,19 @@ def test_data_dependent_problems_are_flagged_not_faulted():
     b2 = dict(b)
     b2["yp"] = b["yp"].copy()
     b2["yp"][1, 1] = 99
-    out = run_device(b2, True)
-    assert out["flags"] & _lib.FLAG_BAD_LABEL
+    for fused in (True, False):
+        out = run_device(b2, fused)
+        assert out["flags"] & _lib.FLAG_BAD_LABEL
+        # the sequence with the bad label cannot be consumed by mistake; the other one is untouched
+        assert np.isnan(out["costs"][1]) and np.isfinite(out["costs"][0])
+        good = run_device(b, fused)
+        assert out["costs"][0] == good["costs"][0]
+    out = run_device(b2, True, with_grad=False)
+    assert np.isnan(out["costs"][1]) and np.isfinite(out["costs"][0])
+    b2c = dict(b2)   # concatenated labels that end too early: the last label of the batch is missing
+    b2c["yc"] = b["yc"][:-1].copy()
+    out = run_device(b2c, True, labels="1d", max_u=3)
+    assert out["flags"] & _lib.FLAG_BAD_LABEL and np.isnan(out["costs"][1]) and np.isfinite(out["costs"][0])
     # lengths that claim more rows than x has
     b3 = dict(b)
     b3["lx"] = np.array([5, 60], dtype=np.int32)
@@ -260,6 +271,30 @@ def test_data_dependent_problems_are_flagged_not_faulted():
         cwarp_rnnt.transducer_loss(b2["x"].to(dev), torch.from_numpy(b2["lx"]).to(dev),
                                    torch.from_numpy(b2["yp"]).to(dev), torch.from_numpy(b2["ly"]).to(dev),
                                    fused_log_softmax=True, validate=True)
+
+
+def test_a_wait_that_runs_out_ends_the_walk_and_poisons_only_its_sequence():
+    """The strips of a sequence wait for each other with bounded polls.  With the bound set to one
+    poll from the host, the second strip of a two-strip sequence gives up at once: the kernel must
+    still finish, flag CWR_FLAG_INTERNAL, give that sequence a NaN cost and leave the one-strip
+    sequences of the batch exact.  With the default bound back, the same batch is exact throughout."""
+    from compactwarprnntloss_amd import _lib
+    lib = _lib.load()
+    b = make_batch([60, 200, 45], [30, 150, 63], 24, seed=8)
+    ref = orc.loss_and_grad(b["x_ref"], b["lx"], b["yp"], b["ly"], 0, "fused", want_dense=False)
+    try:
+        lib.cwr_debug_wait_limit(1)
+        for with_grad in (True, False):
+            out = run_device(b, True, with_grad=with_grad)
+            assert out["flags"] & _lib.FLAG_INTERNAL
+            assert np.isnan(out["costs"][1])
+            np.testing.assert_allclose(out["costs"][[0, 2]], ref["costs"][[0, 2]], rtol=LOSS_RTOL)
+    finally:
+        lib.cwr_debug_wait_limit(0)
+    out = run_device(b, True)
+    assert out["flags"] == 0
+    np.testing.assert_allclose(out["costs"], ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(out["G"], ref["G"], rtol=0, atol=GRAD_ATOL)
 
 
 # ----------------------------------------------------------------------------- golden fixtures

@@ -134,7 +134,26 @@ def test_pack_flags_a_sequence_that_does_not_fit_the_padded_tensor():
     torch.cuda.synchronize()
     assert rc == 0
     assert int(status[0].item()) & 2
-    assert torch.all(out[: 12 + 10] == 1.0) and torch.all(out[12 + 10:] == -7.0)   # frame 5 of sequence 1 is missing
+    # frame 5 of sequence 1 is missing from the padded tensor: its rows are zeroed, never left as they were
+    assert torch.all(out[: 12 + 10] == 1.0) and torch.all(out[12 + 10:] == 0.0)
+    # rows that belong to no sequence (more rows than the lengths add up to) are zeroed as well
+    row_off2, status2 = pkg.loss._offsets(lx, ly, R + 3)
+    xp2 = torch.ones((2, 6, 3, 8), device=DEV)
+    out2 = torch.full((R + 3, 8), -7.0, device=DEV)
+    rc = lib.cwr_pack(xp2.data_ptr(), 0, 2, 6, 3, 8, lx.data_ptr(), ly.data_ptr(), row_off2.data_ptr(), R + 3,
+                      out2.data_ptr(), status2.data_ptr(), None)
+    torch.cuda.synchronize()
+    assert rc == 0 and int(status2[0].item()) & 1
+    assert torch.all(out2[:R] == 1.0) and torch.all(out2[R:] == 0.0)
+    with pytest.raises(RuntimeError):
+        pkg.pack_padded(xp, lx, ly, total_rows=R, validate=True)
+    # the joiner front end behaves the same way
+    f = torch.ones((2, 5, 16), device=DEV)
+    g = torch.ones((2, 3, 16), device=DEV)
+    h = pkg.compact_join(f, g, lx, ly, None, total_rows=R)
+    assert torch.all(h[: 12 + 10] == 2.0) and torch.all(h[12 + 10:] == 0.0)
+    with pytest.raises(RuntimeError):
+        pkg.compact_join(f, g, lx, ly, "tanh", total_rows=R, validate=True)
 
 
 @pytest.mark.parametrize("fused", [True, False])
