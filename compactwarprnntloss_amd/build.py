@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libcwarp_rnnt_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["api.hip", "lattice.hip", "rows.hip", "pack.hip", "join.hip"]
+SOURCES = ["api.hip", "lattice.hip", "rows.hip", "pack.hip", "join.hip", "joint.hip"]
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off: hipcc would otherwise pair fp32 operations into packed
 # instructions, which have produced sporadic wrong results on the target machines.
@@ -53,7 +53,7 @@ def build(verbose: bool = True) -> str:
             print(err, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp]

@@ -228,8 +228,9 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
                         int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse, float* grads,
-                        float* costs, float* reduced, void* stream, bool with_grad) {
-    int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+                        float* costs, float* reduced, void* stream, bool with_grad,
+                        const JointOperands* joint = nullptr) {
+    int rc = check_common(x, joint == nullptr, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
     if (rc != CWR_OK) return rc;
     if (max_u < 0) return CWR_ERR_SHAPE;
     if (!row_off || !lab_off || !status) return CWR_ERR_NULL;
@@ -251,7 +252,8 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
-    rc = launch_gather(b, ws, lse, rowinfo, with_grad ? grads : nullptr);
+    rc = joint ? launch_joint_gather(b, ws, *joint, lse, rowinfo, with_grad ? grads : nullptr)
+               : launch_gather(b, ws, lse, rowinfo, with_grad ? grads : nullptr);
     if (rc != CWR_OK) return rc;
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;
@@ -283,6 +285,23 @@ int cwr_forward_noalloc(const void* x, int dtype, int64_t R, int64_t V, const in
     if (rc != CWR_OK) return rc;
     return forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, ws, need, row_off,
                         lab_off, status, rowinfo, lse, grads, costs, nullptr, stream, true);
+}
+
+int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                      const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                      int64_t N, int32_t blank, int64_t max_u, void* workspace, size_t workspace_bytes_,
+                      int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
+                      float* grads, float* costs, void* stream) {
+    if (dtype != CWR_F16 && dtype != CWR_BF16) return CWR_ERR_DTYPE;
+    if (H < 32 || H % 32 != 0) return CWR_ERR_SHAPE;  // K-slices of 32
+    if (H > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (R > 0 && (!h || !w)) return CWR_ERR_NULL;
+    if (misaligned(h, 16) || misaligned(w, 16) || misaligned(bias, 4)) return CWR_ERR_ALIGN;
+    JointOperands j;
+    j.h = h; j.w = w; j.bias = bias; j.H = H;
+    return forward_impl(nullptr, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, CWR_MODE_FUSED, max_u, workspace,
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream, true,
+                        &j);
 }
 
 int cwr_forward_reduced(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,

@@ -291,4 +291,48 @@ __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restr
     return lab;
 }
 
+// What the lattice walk consumes, one 16-byte record per cell (see LpCell): the (blank, label)
+// log-probabilities as base-2 logarithms, floored so that -inf logits stay finite, and the same
+// two as plain probabilities for the scaled linear-domain walk.  A logarithm outside
+// [kLinMin, kLinMax] cannot be carried by that walk within one of its blocks (nor, as a
+// probability, by fp32); the sequence is then marked for the log-domain walk.
+// A row's log-sum-exp as (maximum m, log2 of the sum of exp(x - m)).  Kept in two parts for the
+// cell records: x - m is exact and log2(sum) is small when a row is peaked, so that a
+// log-probability close to zero keeps its absolute accuracy however large the logits are (one
+// fp32 number m + ln(sum) would carry half an ulp of m into every log-probability).
+struct Lse {
+    float m, l2s;
+    __device__ __forceinline__ float value() const { return fmaf(l2s, kLn2, m); }
+};
+// log2 of a sum s >= 1 of exponentials whose largest term is 1, and 2^b for a log-probability b:
+// series next to s = 1 and b = 0, where the hardware approximations are good to an ulp of their
+// RESULT's neighbourhood (about 1e-7 absolute) but a peaked row needs the small difference itself.
+__device__ __forceinline__ float log2_of_sum(float s) {
+    const float d = s - 1.f;  // exact for s in [1, 2]
+    const float series = d * fmaf(d, fmaf(d, 1.f / 3.f, -0.5f), 1.f) * kLog2e;
+    return d < 0.015625f ? series : fast_log2(s);
+}
+__device__ __forceinline__ float exp2_of_logprob(float b) {
+    const float z = b * kLn2;
+    const float series = fmaf(z, fmaf(z, fmaf(z, 1.f / 6.f, 0.5f), 1.f), 1.f);
+    return b > -0.015625f ? series : fast_exp2(b);
+}
+
+// lab: the row's label, kNoLabel or kBadLabel.  The walk-mode word is looked at before it is set: a
+// batch of steep logits marks its sequences from most rows at once, and unconditional atomics on one
+// address per sequence would queue.
+__device__ __forceinline__ LpCell make_lp(float xb, float xl, const Lse lse, int lab, int* seqmode_n) {
+    const float b = (float)(((double)fmaxf(xb, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s);
+    const float l = lab >= 0
+        ? (float)(((double)fmaxf(xl, kLpFloor) - (double)lse.m) * 1.4426950408889634 - (double)lse.l2s) : 0.f;
+    if (!(b >= kLinMin && b <= kLinMax && l >= kLinMin && l <= kLinMax)) raise_flag(seqmode_n, kSeqLogDomain);
+    if (lab == kBadLabel) raise_flag(seqmode_n, kSeqPoisoned);
+    LpCell c;
+    c.p_blank = exp2_of_logprob(b);
+    c.p_label = exp2_of_logprob(l);
+    c.l_blank = b;
+    c.l_label = l;
+    return c;
+}
+
 }  // namespace cwr

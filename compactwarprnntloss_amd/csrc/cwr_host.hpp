@@ -62,6 +62,16 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 // grads (may be null): rows of skipped sequences get a zero record there
 int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads);
 int launch_rowinfo(const Batch& b, int* rowinfo);
+// The fused output layer: logits = h (R,H) x W^T (V,H) + bias, never stored.  b.dtype is the type of
+// h and W (CWR_F16 or CWR_BF16), b.V the vocabulary, b.x unused.
+struct JointOperands {
+    const void* h;
+    const void* w;
+    const float* bias;  // may be null
+    i64 H;
+};
+int launch_joint_gather(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
+                        float* grads);
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only);
 // reduced (may be null): 2 floats, sum and mean of the N costs
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs,

@@ -116,6 +116,56 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     return costs, st
 
 
+def joint_forward(h, weight, bias, lx, ys, ly, blank: int, max_u: Optional[int] = None):
+    """Binding of cwr_joint_forward: the loss of logits = h @ weight.T + bias without ever storing
+    them.  h (R,H) and weight (V,H) fp16 or bf16, bias (V,) or None.  Returns (costs fp32 (N,),
+    ForwardState) like rnnt_forward in fused mode."""
+    if h.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != h.dtype:
+        raise RuntimeError("h and weight must both be float16 or both bfloat16")
+    if h.dim() != 2 or weight.dim() != 2 or h.size(1) != weight.size(1):
+        raise RuntimeError("h must be (R, H) and weight (V, H)")
+    if h.size(1) % 32 != 0:
+        raise RuntimeError("the joint dimension must be a multiple of 32")
+    if not weight.is_cuda or not weight.is_contiguous():
+        raise RuntimeError("weight must be a contiguous CUDA tensor")
+    _check_inputs(h, lx, ys, ly)
+    lib = _lib.load()
+    dev = h.device
+    N = lx.numel()
+    R, H = h.shape
+    V = weight.size(0)
+    y_stride, y_len = _label_args(ys)
+    if max_u is None:
+        max_u = ys.size(1) if ys.dim() == 2 else (int(ly.max().item()) if ly.numel() else 0)
+    b32 = None
+    if bias is not None:
+        if bias.numel() != V:
+            raise RuntimeError("bias must hold one value per vocabulary entry")
+        b32 = bias.detach().to(dtype=torch.float32).contiguous()
+    st = ForwardState()
+    st.N, st.R, st.V, st.mode, st.max_u = N, R, V, _lib.MODE_FUSED, int(max_u)
+    meta = torch.empty(2 * (N + 1) + 2, dtype=torch.int64, device=dev)
+    st.row_off = meta[: N + 1]
+    st.lab_off = meta[N + 1: 2 * (N + 1)]
+    st.status = meta[2 * (N + 1):].view(torch.int32)
+    ws_bytes = lib.cwr_workspace_bytes(N, R, int(max_u))
+    st.workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    costs = torch.empty(N, dtype=torch.float32, device=dev)
+    st.reduced = None
+    st.lse = torch.empty(R, dtype=torch.float32, device=dev)
+    st.grads = torch.empty((R, 2), dtype=torch.float32, device=dev)
+    st.rowinfo = torch.empty((R, 2), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = lib.cwr_joint_forward(h.data_ptr(), weight.data_ptr(), b32.data_ptr() if b32 is not None else None,
+                                   _DTYPES[h.dtype], R, H, V, lx.data_ptr(), ly.data_ptr(), ys.data_ptr(), y_stride,
+                                   y_len, N, int(blank), int(max_u), st.workspace.data_ptr(), ws_bytes,
+                                   st.row_off.data_ptr(), st.lab_off.data_ptr(), st.status.data_ptr(),
+                                   st.rowinfo.data_ptr(), st.lse.data_ptr(), st.grads.data_ptr(), costs.data_ptr(),
+                                   _stream_ptr(dev))
+        _lib.check(rc, "cwr_joint_forward")
+    return costs, st
+
+
 def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torch.Tensor,
                   out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
     """Binding of cwr_backward.  Returns the (R,V) gradient in xs.dtype.

@@ -275,6 +275,25 @@ int cwr_join_backward(const void* dh, const void* h, int dtype, int act, int64_t
                       int64_t H, const int32_t* lx, const int32_t* ly, const int64_t* row_off, int64_t R, void* df,
                       void* dg, void* stream);
 
+/* cwr_forward for logits that are never stored: the joiner's output layer
+ * logits[r, v] = sum_k h[r, k] * w[v, k] + bias[v] is multiplied tile by tile on the matrix cores
+ * (16-bit inputs, fp32 accumulation) and every tile is reduced on the spot to what the loss needs
+ * of a row: its log-sum-exp over V and its blank and label logits.  The reference repository has
+ * no joiner; this replaces, for its callers, the output-layer GEMM, the log-softmax
+ * (test/test.py:19-20) and the gather pass (cwarp_cuda_gather_kernel.cu:19-43) that cwr_forward in
+ * CWR_MODE_FUSED would run on stored logits, and removes the (R, V) logits from memory.
+ *   h     (R, H) compact joint activations (e.g. from cwr_join), w (V, H) output-layer weight (the
+ *         layout of a torch.nn.Linear weight), both of `dtype` = CWR_F16 or CWR_BF16, contiguous,
+ *         16-byte aligned;  H a multiple of 32
+ *   bias  (V,) fp32 or NULL
+ * All other arguments and every output as for cwr_forward with mode = CWR_MODE_FUSED; lse, rowinfo
+ * and grads are what cwr_joint_backward reads. */
+int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                      const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                      int64_t N, int32_t blank, int64_t max_u, void* workspace, size_t workspace_bytes,
+                      int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
+                      float* grads, float* costs, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -140,6 +140,23 @@ def join_rows_backward(dh, f, g, lx, ly, act=None):
     return df, dg
 
 
+def joint_logits(h, w, bias=None):
+    """Output layer of a joiner in float64: logits[r, v] = sum_k h[r, k] * w[v, k] + bias[v], for
+    compact joint activations h (R, H) and a weight w (V, H) laid out as torch.nn.Linear keeps it.
+    (The reference repository has no joiner; its callers feed such logits, after log_softmax, to
+    cwarp_rnnt/__init__.py:32-73, test/test.py:19-20.)"""
+    z = np.asarray(h, dtype=np.float64) @ np.asarray(w, dtype=np.float64).T
+    if bias is not None:
+        z = z + np.asarray(bias, dtype=np.float64)[None, :]
+    return z
+
+
+def joint_backward(dlogits, h, w):
+    """Backward of joint_logits: (dh (R,H), dw (V,H), dbias (V,)) for dlogits (R,V)."""
+    d = np.asarray(dlogits, dtype=np.float64)
+    return d @ np.asarray(w, dtype=np.float64), d.T @ np.asarray(h, dtype=np.float64), d.sum(axis=0)
+
+
 def labels_of(y, ly, n):
     """Labels of sequence n from either padded (N,Umax) or concatenated (sum U,) labels."""
     y = np.asarray(y)
