@@ -19,8 +19,6 @@
 // cross-lane traffic until the very end.  Waves split the tile 2 x 2: wave (wd, wv) multiplies the
 // data rows [128 wd, 128 wd + 128) with the vocabulary entries [64 wv, 64 wv + 64) of the tile.
 #include "cwr_device.hpp"
-#include <cstdlib>
-
 #include "cwr_host.hpp"
 
 namespace cwr {
@@ -283,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void k_joint_fwd(
 constexpr int kRK = 64;      // K-slice of the weight tile
 constexpr int kRPitch = 72;  // 144 bytes: 16 consecutive rows start in 16 different groups of four banks
 
-template <typename T, int ND, int KS /* H / 16 */, int OCC>
+template <typename T, int ND, int KS /* H / 16 */, int OCC, bool D2>
 __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
     const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
@@ -327,7 +325,7 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     // ---- weight tile: thread t moves 16-byte piece (t % 8) of rows t / 8 + 32 p, p = 0..3 ----------
     const int st_row = tid >> 3, st_piece = tid & 7;
     struct Pre { v4i w[4]; };
-    Pre pre[2];
+    Pre pre[D2 ? 2 : 1];
     const int nvt = (V + kJN - 1) / kJN;
     auto fetch = [&](int vt, int kc, Pre& q) {
 #pragma unroll
@@ -357,7 +355,7 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     float bias_next = 0.f;
     if (tid < kJN) s_bias[0][tid] = bias_of(0);
     fetch(0, 0, pre[0]);
-    if (NK > 1 || nvt > 1) fetch(NK > 1 ? 0 : 1, NK > 1 ? 1 : 0, pre[1]);
+    if (D2 && (NK > 1 || nvt > 1)) fetch(NK > 1 ? 0 : 1, NK > 1 ? 1 : 0, pre[1]);
     stage(0, pre[0]);
     __syncthreads();
 
@@ -381,27 +379,36 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
         for (int kc = 0; kc < NK; ++kc) {
             if (kc == NK - 1 && tid < kJN && vt + 1 < nvt) s_bias[(vt + 1) & 1][tid] = bias_next;  // before its barrier
             // register set kc & 1 held this slice's loads (already staged); it now takes slice it + 2
-            {
+            if (D2) {
                 const int k2 = kc + 2;
                 const int vt2 = vt + k2 / NK, kc2 = k2 % NK;
                 if (vt2 < nvt) fetch(vt2, kc2, pre[(kc + (NK & 1) * vt) & 1]);
+            } else {
+                const int k1 = kc + 1;
+                const int vt1 = vt + k1 / NK, kc1 = k1 % NK;
+                if (vt1 < nvt) fetch(vt1, kc1, pre[0]);
             }
+            // The four weight fragments of a K-step are requested together and the matrix
+            // instructions follow as they arrive (left to itself the compiler reuses ONE fragment
+            // register and pays the LDS latency in front of every matrix instruction).
 #pragma unroll
             for (int ks = 0; ks < kRK / 16; ++ks) {
                 v4i fa[4];
 #pragma unroll
                 for (int mv = 0; mv < 4; ++mv)
                     fa[mv] = *reinterpret_cast<const v4i*>(&s_w[par][32 * mv + l32][16 * ks + 8 * hf]);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int mv = 0; mv < 4; ++mv)
 #pragma unroll
                     for (int nd = 0; nd < ND; ++nd)
                         acc[mv][nd] = Mfma<T>::mac(fa[mv], hreg[nd][kc * (kRK / 16) + ks], acc[mv][nd]);
+                __builtin_amdgcn_sched_barrier(0);
             }
             {
                 const int k1 = kc + 1;
                 const int vt1 = vt + k1 / NK;
-                if (vt1 < nvt) stage(par ^ 1, pre[(kc + 1 + (NK & 1) * vt) & 1]);
+                if (vt1 < nvt) stage(par ^ 1, pre[D2 ? (kc + 1 + (NK & 1) * vt) & 1 : 0]);
             }
             __syncthreads();
             par ^= 1;
@@ -464,14 +471,6 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     }
 }
 
-// experiment switch: CWR_JOINT_VARIANT = "<ND><OCC>" picks among the instantiations of one H
-static bool variant_ok(int nd, int occ) {
-    const char* e = getenv("CWR_JOINT_VARIANT");
-    if (!e || !e[0]) return true;
-    if (e[0] == 's') return false;
-    return e[0] - '0' == nd && e[1] - '0' == occ;
-}
-
 template <typename T>
 static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
                               float* grads) {
@@ -479,18 +478,20 @@ static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOp
     float2* gz = reinterpret_cast<float2*>(grads);
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
-#define CWR_JOINT_RES(ND, KS, OCC)                                                                              \
-    if (j.H == 16 * KS && variant_ok(ND, OCC)) {                                                                                       \
+#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                              \
+    if (j.H == 16 * KS) {                                                                                       \
         const i64 blocks = (b.R + 128 * ND - 1) / (128 * ND);                                                   \
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                    \
-        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, OCC>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w, j.bias,  \
+        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w, j.bias,  \
                    b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,       \
                    b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);                                          \
         return check_launch();                                                                                  \
     }
     // the joint sizes in use; any other multiple of 32 takes the streaming kernel
-    CWR_JOINT_RES(2, 16, 1) CWR_JOINT_RES(2, 24, 1) CWR_JOINT_RES(2, 32, 1) CWR_JOINT_RES(1, 32, 1) CWR_JOINT_RES(1, 32, 2)
-    CWR_JOINT_RES(1, 40, 1) CWR_JOINT_RES(1, 48, 1) CWR_JOINT_RES(1, 64, 1)
+    // measured on R = 311449, V = 1024, H = 512 (bf16): one data block per wave at two waves per SIMD
+    // 0.46 ms; two blocks per wave at one wave per SIMD 0.63 ms (registers spill); streaming kernel 0.63 ms
+    CWR_JOINT_RES(2, 16, 1, true) CWR_JOINT_RES(2, 24, 1, true) CWR_JOINT_RES(1, 32, 2, false)
+    CWR_JOINT_RES(1, 40, 1, true) CWR_JOINT_RES(1, 48, 1, true) CWR_JOINT_RES(1, 64, 1, true)
 #undef CWR_JOINT_RES
     const i64 blocks = (b.R + kJM - 1) / kJM;
     if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
