@@ -29,6 +29,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16 matrix-core peak of MI355X
 WORKLOADS = {
     1: "c1 tiny: N=4 T~U[8,32] U~U[2,10] V=32 fp32",
     2: "c2 BPE ASR: N=32 T~U[100,250] U~U[20,80] V=1024 fp32 logits N(0,2), blank=0, mean reduction",
@@ -96,6 +97,10 @@ def main():
     ap.add_argument("--with-pack", action="store_true",
                     help="also time the padded -> compact pack op and its backward on the padded form of the same "
                          "batch (reported under 'pack_op'; not part of 'value')")
+    ap.add_argument("--with-fused-joiner", action="store_true",
+                    help="also time the output layer fused into the loss (cwr_joint_forward / cwr_joint_backward) "
+                         "against the route through stored logits")
+    ap.add_argument("--joint-dim", type=int, default=512, help="H of --with-fused-joiner")
     ap.add_argument("--with-joiner", action="store_true",
                     help="also time the compact joiner front (broadcast sum + tanh for valid cells, H=512, in the "
                          "batch's storage type) and its backward at the same lengths (reported under 'joiner_op'; "
@@ -267,6 +272,67 @@ def main():
                          "backward_GBs": round((2 if act == 0 else 4) * rb / (bw * 1e-3) / 1e9, 1)}
         result["joiner_op"] = {"H": H, "rows": R, **ops}
         del f, g, h, dh, df, dg
+
+    if args.with_fused_joiner:
+        # The output layer fused into the loss (cwr_joint_forward / cwr_joint_backward) on this config's
+        # lengths: bf16 (R,H) x (H,V) on the matrix cores.  Algorithmic flops: 2 R H V forward, 6 R H V
+        # forward + backward (logits, dh, dW); the logits formed a second time in the backward pass
+        # are not counted.  Beside it the route through stored logits: library GEMM, then the fused
+        # loss over the (R,V) bf16 logits (three passes over them).
+        H = args.joint_dim
+        jd = torch.bfloat16
+        hj = torch.randn((R, H), device=dev).to(jd)
+        Wj = (torch.randn((V, H), device=dev) / H ** 0.5).to(jd)
+        bj = torch.randn(V, device=dev).to(jd)
+        lib = pkg._lib.load()
+        stream = torch.cuda.current_stream().cuda_stream
+        flops = 2.0 * R * H * V
+        fwd_call = timed(lambda: pkg.joint_forward(hj, Wj, bj, lx, y, ly, 0, max_u=y.size(1)))
+        _c, jst = pkg.joint_forward(hj, Wj, bj, lx, y, ly, 0, max_u=y.size(1))
+        b32 = bj.float()
+        dzb = torch.empty((R, V), dtype=jd, device=dev)
+        dz_ms = timed(lambda: lib.cwr_joint_backward(
+            hj.data_ptr(), Wj.data_ptr(), b32.data_ptr(), pkg.loss._DTYPES[jd], R, H, V, N, 0, jst.rowinfo.data_ptr(),
+            jst.grads.data_ptr(), jst.lse.data_ptr(), go.data_ptr(), 1, 1.0, dzb.data_ptr(), stream))
+        del dzb, jst
+        hp, Wp, bp = (t.clone().requires_grad_(True) for t in (hj, Wj, bj))
+
+        def fused_step():
+            hp.grad = Wp.grad = bp.grad = None
+            pkg.fused_joint_loss(hp, Wp, bp, lx, y, ly, 0, "mean", max_u=y.size(1)).backward()
+
+        def stored_step():
+            hp.grad = Wp.grad = bp.grad = None
+            z = torch.nn.functional.linear(hp, Wp, bp)
+            pkg.transducer_loss(z, lx, y, ly, 0, "mean", fused_log_softmax=True, max_u=y.size(1)).backward()
+
+        def stored_fwd():
+            with torch.no_grad():
+                z = torch.nn.functional.linear(hj, Wj, bj)
+            pkg.rnnt_forward(z, lx, y, ly, 0, True, max_u=y.size(1))
+
+        torch.cuda.reset_peak_memory_stats()
+        base_mem = torch.cuda.memory_allocated()
+        fused_ms = timed(fused_step)
+        fused_mem = torch.cuda.max_memory_allocated() - base_mem
+        torch.cuda.reset_peak_memory_stats()
+        stored_ms = timed(stored_step)
+        stored_mem = torch.cuda.max_memory_allocated() - base_mem
+        stored_fwd_ms = timed(stored_fwd)
+        result["fused_joiner"] = {
+            "H": H, "rows": R, "V": V, "dtype": "bf16", "peak_TFLOPs": MFMA_BF16_PEAK_TFLOPS,
+            "forward_call_ms": round(fwd_call, 4),
+            "forward_TFLOPs": round(flops / (fwd_call * 1e-3) / 1e12, 1),
+            "dlogits_kernel_ms": round(dz_ms, 4),
+            "dlogits_TFLOPs": round(flops / (dz_ms * 1e-3) / 1e12, 1),
+            "fwd_bwd_ms": round(fused_ms, 4),
+            "fwd_bwd_TFLOPs": round(3 * flops / (fused_ms * 1e-3) / 1e12, 1),
+            "fwd_bwd_frac_of_peak": round(3 * flops / (fused_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "fwd_bwd_peak_extra_MiB": round(fused_mem / 2 ** 20, 1),
+            "stored_logits_route": {"what": "torch linear (library GEMM) + transducer_loss(fused_log_softmax=True)",
+                                    "forward_ms": round(stored_fwd_ms, 4), "fwd_bwd_ms": round(stored_ms, 4),
+                                    "fwd_bwd_peak_extra_MiB": round(stored_mem / 2 ** 20, 1)}}
+        del hj, Wj, bj, hp, Wp, bp
 
     if not args.no_cpu:
         g_all = pkg.rnnt_backward(xd, lx, y, ly, 0, st, go, out=out)

@@ -304,6 +304,28 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
                         &j);
 }
 
+int cwr_joint_backward(const void* h, const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                       int64_t N, int32_t blank, const int32_t* rowinfo, const float* grads, const float* lse,
+                       const float* grad_costs, int64_t grad_stride, float grad_scale, void* dlogits, void* stream) {
+    if (dtype != CWR_F16 && dtype != CWR_BF16) return CWR_ERR_DTYPE;
+    if (R < 0 || N < 0 || V < 1) return CWR_ERR_SHAPE;
+    if (H < 32 || H % 32 != 0) return CWR_ERR_SHAPE;  // K-slices of 32
+    if (H > 0x3fffffff || V > 0x3fffffff || N > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (blank < 0 || blank >= V) return CWR_ERR_BLANK;
+    if (grad_stride != 0 && grad_stride != 1) return CWR_ERR_SHAPE;
+    if (R == 0) return CWR_OK;
+    if (!h || !w || !rowinfo || !grads || !lse || !grad_costs || !dlogits) return CWR_ERR_NULL;
+    if (misaligned(h, 16) || misaligned(w, 16) || misaligned(bias, 4) || misaligned(rowinfo, 8) ||
+        misaligned(grads, 8) || misaligned(lse, 4) || misaligned(grad_costs, 4) ||
+        misaligned(dlogits, (V & 3) == 0 ? 8 : 2))  // runs of four entries leave as 8-byte stores
+        return CWR_ERR_ALIGN;
+    JointOperands j;
+    j.h = h; j.w = w; j.bias = bias; j.H = H;
+    const GradOut go = {grad_costs, grad_stride, grad_scale};
+    return launch_joint_dlogits(dtype, j, R, V, N, blank, rowinfo, grads, lse, go, dlogits,
+                                static_cast<hipStream_t>(stream));
+}
+
 int cwr_forward_reduced(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,

@@ -86,6 +86,10 @@ struct GradOut {
 int launch_grad(const Batch& b, const int* rowinfo, const float* grads, const float* lse,
                 const GradOut grad_costs, void* grad_x);
 
+// d loss / d logits of the rows [0, R) of a block, from logits formed again on the matrix cores
+int launch_joint_dlogits(int dtype, const JointOperands& j, i64 R, i64 V, i64 N, int blank, const int* rowinfo,
+                         const float* grads, const float* lse, const GradOut go, void* dlogits, hipStream_t stream);
+
 int launch_export(const int* lx, const int* ly, int N, i64 T_pad, i64 Up_pad, const Workspace& ws,
                   double* alphas_out, double* betas_out, hipStream_t stream);
 int launch_repack(const void* src, void* dst, size_t esize, const int* lx, const int* ly, const i64* row_off, i64 N,

@@ -6,6 +6,11 @@
 //             i.e. exactly what the gather pass of the loss (cwarp_cuda_gather_kernel.cu:19-43 plus
 //             the log-softmax the reference's callers run first, test/test.py:19-20) extracts from
 //             stored logits; the lattice then runs as usual.
+//   backward  k_joint_dz: the same tiles are formed again and turned, in registers, into
+//             d loss / d logits = softmax * gamma + [blank] + [label] terms (what the gradient pass of
+//             the loss would write from stored logits, cwarp_cuda_gather_kernel.cu:52-74 plus the
+//             log-softmax backward), rounded once to the 16-bit type and written for a block of rows
+//             at a time; the caller multiplies that block into dh, dW and dbias and reuses the buffer.
 //
 // The reference repository has no joiner; its callers hand stored logits to
 // cwarp_rnnt/__init__.py:32-73.
@@ -61,37 +66,27 @@ __device__ __forceinline__ void lse_merge(float& m, float& s, float m2, float s2
 // entry, for a lane of half `hf` = lane / 32 (the block's data row is lane % 32).
 __device__ __forceinline__ constexpr int acc_row(int r, int hf) { return 8 * (r >> 2) + 4 * hf + (r & 3); }
 
-template <typename T>
-__global__ __launch_bounds__(256, 2) void k_joint_fwd(
-    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int H, int V,
-    const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
-    const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
-    int blank, LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
-    __shared__ __attribute__((aligned(16))) T s_h[2][kJM][kJPitch];
-    __shared__ __attribute__((aligned(16))) T s_w[2][kJN][kJPitch];
-    __shared__ __attribute__((aligned(16))) float s_bias[2][kJN];  // what the accumulators of a tile start from
+// The walk of the streaming kernels: every complete tile of logits is handed to
+// tile(acc, first vocabulary entry of this wave's part); acc[mv][nd] is the 32x32 block of vocabulary
+// entries [32 mv, 32 mv + 32) of the wave's part and data rows [32 nd, 32 nd + 32) of its 128.
+template <typename T> struct StreamLds {
+    T h[2][kJM][kJPitch];
+    T w[2][kJN][kJPitch];
+    float bias[2][kJN];  // what the accumulators of a tile start from
+};
 
+template <typename T, typename TileFn>
+__device__ __forceinline__ void walk_streaming(const T* __restrict__ h, const T* __restrict__ W,
+                                               const float* __restrict__ bias, i64 R, int H, int V, i64 row0,
+                                               StreamLds<T>& lds, TileFn&& tile) {
+    auto& s_h = lds.h;
+    auto& s_w = lds.w;
+    auto& s_bias = lds.bias;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wd = w & 1, wv = w >> 1;
     const int hf = lane >> 5, l32 = lane & 31;
-    const i64 row0 = (i64)blockIdx.x * kJM;
-
-    // ---- the rows this lane reduces: data rows row0 + 128 wd + 32 nd + l32, nd = 0..3 ----------
-    // (only the label is needed during the walk over the vocabulary; the row's place in its lattice
-    // is worked out again at the end rather than kept in registers all along)
-    int lab[4];
-#pragma unroll
-    for (int nd = 0; nd < 4; ++nd) {
-        const i64 r = row0 + 128 * wd + 32 * nd + l32;
-        lab[nd] = kNoLabel;
-        if (r < R) {
-            const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-            if (ri.n >= 0 && pad_off[ri.n] >= 0) lab[nd] = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-        }
-    }
 
     // ---- global -> LDS staging: thread t moves 16-byte piece (t % 4) of rows t / 4 + 64 p ----------
     // The loads of a K-slice are issued TWO slices ahead of its use (two register sets taking turns):
@@ -126,12 +121,6 @@ __global__ __launch_bounds__(256, 2) void k_joint_fwd(
 #pragma unroll
         for (int p = 0; p < 2; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + 64 * p][st_piece * 8]) = q.w[p];
     };
-
-    // running log-sum-exp state of the lane's rows over the vocabulary entries it has seen, and
-    // the two logits the loss wants
-    float m[4], s[4], xl[4], xb[4];
-#pragma unroll
-    for (int nd = 0; nd < 4; ++nd) { m[nd] = -INFINITY; s[nd] = 0.f; xl[nd] = 0.f; xb[nd] = 0.f; }
 
     // the bias of a tile (-inf beyond the vocabulary, which no finite product changes and which drops
     // out of both the maximum and the sum) is fetched by the first 128 threads one tile ahead
@@ -189,88 +178,295 @@ __global__ __launch_bounds__(256, 2) void k_joint_fwd(
         __syncthreads();
         if (kc != nk - 1) return;
 
-        // ---- the tile's logits are complete: fold them into the rows' running state ----------
-        const int blank_key = (blank >= v_wave && blank < v_wave + 64 && (((blank - v_wave) >> 2) & 1) == hf)
-                                  ? blank - v_wave : -1;
-#pragma unroll
-        for (int nd = 0; nd < 4; ++nd) {
-            float mx = acc[0][nd][0];
-#pragma unroll
-            for (int mv = 0; mv < 2; ++mv)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[mv][nd][r]);
-            const float mn = fmaxf(m[nd], mx);
-            if (mn > -INFINITY) {
-                const float ms = mn * kLog2e;
-                float sum = s[nd] * fast_exp2(fmaf(m[nd], kLog2e, -ms));  // m = -inf: s = 0 stays 0
-#pragma unroll
-                for (int mv = 0; mv < 2; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sum += fast_exp2(fmaf(acc[mv][nd][r], kLog2e, -ms));
-                s[nd] = sum;
-                m[nd] = mn;
-            }
-            // the label's logit, if it sits in this lane's half of this wave's part of the tile
-            const int lv = lab[nd] - v_wave;
-            const int key = (lab[nd] >= 0 && lv >= 0 && lv < 64 && ((lv >> 2) & 1) == hf) ? lv : -1;
-            if (__ballot(key >= 0) != 0) {
-#pragma unroll
-                for (int mv = 0; mv < 2; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) xl[nd] = key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : xl[nd];
-            }
-            if (__ballot(blank_key >= 0) != 0) {
-#pragma unroll
-                for (int mv = 0; mv < 2; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        xb[nd] = blank_key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : xb[nd];
-            }
-        }
+        tile(acc, v_wave);
     };
     for (int it = 0; it < iters; it += 2) {
         slice(it, pre[0], pre[1]);
         if (it + 1 < iters) slice(it + 1, pre[1], pre[0]);
     }
 
+}
+
+// ---------------------------------------------------------------------------------------------
+// what the forward kernels do with a finished tile
+// ---------------------------------------------------------------------------------------------
+// Per lane and data row: the running (maximum, sum of exponentials) over the vocabulary entries the
+// lane has seen, and the two logits the loss wants (0 until seen; exactly one lane sees each).
+template <int ND> struct FwdRows {
+    float m[ND], s[ND], xl[ND], xb[ND];
+    int lab[ND];
+};
+
+template <int ND>
+__device__ __forceinline__ void fwd_rows_init(FwdRows<ND>& q, i64 rbase, i64 R, const int* __restrict__ lx,
+                                              const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride,
+                                              i64 y_len, const i64* __restrict__ row_off,
+                                              const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
+                                              int V, int* __restrict__ status) {
+    // (only the label is needed during the walk over the vocabulary; the row's place in its lattice
+    // is worked out again at the end rather than kept in registers all along)
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        q.m[nd] = -INFINITY; q.s[nd] = 0.f; q.xl[nd] = 0.f; q.xb[nd] = 0.f;
+        const i64 r = rbase + 32 * nd;
+        q.lab[nd] = kNoLabel;
+        if (r < R) {
+            const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+            if (ri.n >= 0 && pad_off[ri.n] >= 0) q.lab[nd] = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
+        }
+    }
+}
+
+// acc[mv][nd]: vocabulary entries v_first + 32 mv + acc_row(., hf) of the lane's data row nd
+template <int NMV, int ND>
+__device__ __forceinline__ void fwd_fold_tile(const f32x16 (&acc)[NMV][ND], int v_first, int blank, int hf,
+                                              FwdRows<ND>& q) {
+    constexpr int SPAN = 32 * NMV;
+    const int blank_key = (blank >= v_first && blank < v_first + SPAN && (((blank - v_first) >> 2) & 1) == hf)
+                              ? blank - v_first : -1;
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        float mx = acc[0][nd][0];
+#pragma unroll
+        for (int mv = 0; mv < NMV; ++mv)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[mv][nd][r]);
+        const float mn = fmaxf(q.m[nd], mx);
+        if (mn > -INFINITY) {
+            const float ms = mn * kLog2e;
+            float sum = q.s[nd] * fast_exp2(fmaf(q.m[nd], kLog2e, -ms));  // m = -inf: s = 0 stays 0
+#pragma unroll
+            for (int mv = 0; mv < NMV; ++mv)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum += fast_exp2(fmaf(acc[mv][nd][r], kLog2e, -ms));
+            q.s[nd] = sum;
+            q.m[nd] = mn;
+        }
+        // the label's logit, if it sits in this lane's half of this part of the tile
+        const int lv = q.lab[nd] - v_first;
+        const int key = (q.lab[nd] >= 0 && lv >= 0 && lv < SPAN && ((lv >> 2) & 1) == hf) ? lv : -1;
+        if (__ballot(key >= 0) != 0) {
+#pragma unroll
+            for (int mv = 0; mv < NMV; ++mv)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) q.xl[nd] = key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : q.xl[nd];
+        }
+        if (__ballot(blank_key >= 0) != 0) {
+#pragma unroll
+            for (int mv = 0; mv < NMV; ++mv)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    q.xb[nd] = blank_key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : q.xb[nd];
+        }
+    }
+}
+
+// the two halves of a wave hold disjoint vocabulary entries of the same rows
+template <int ND> __device__ __forceinline__ void fwd_merge_halves(FwdRows<ND>& q) {
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        lse_merge(q.m[nd], q.s[nd], __shfl_xor(q.m[nd], 32), __shfl_xor(q.s[nd], 32));
+        q.xl[nd] += __shfl_xor(q.xl[nd], 32);  // exactly one half held the entry, the other 0
+        q.xb[nd] += __shfl_xor(q.xb[nd], 32);
+    }
+}
+
+struct FwdOut {
+    LpCell* lp;
+    float* lse;
+    int2* rowinfo;
+    float2* grads_skipped;
+    int* seqmode;
+};
+
+__device__ __forceinline__ void fwd_row_out(i64 r, i64 R, float m, float s, float xb, float xl, int lab,
+                                            const int* __restrict__ lx, const int* __restrict__ ly,
+                                            const i64* __restrict__ row_off, const i64* __restrict__ pad_off, int N,
+                                            const FwdOut& o) {
+    const Lse lse = {m, log2_of_sum(s)};
+    o.lse[r] = lse.value();
+    const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
+    const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
+    o.rowinfo[r] = make_int2(lab < 0 ? -1 : lab, ri.n);
+    if (pad >= 0)
+        o.lp[pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1)] = make_lp(xb, xl, lse, lab, o.seqmode + ri.n);
+    else if (o.grads_skipped) o.grads_skipped[r] = make_float2(0.f, 0.f);
+}
+
+// ---------------------------------------------------------------------------------------------
+// what the backward kernels do with a finished tile
+// ---------------------------------------------------------------------------------------------
+// Per lane and data row the coefficients of
+//   dz[r, v] = softmax(z_r)[v] * cg + [v == blank] * cb + [v == label] * cl,   softmax = 2^(z log2 e + nls)
+// i.e. cwr_backward's CWR_MODE_FUSED formula on logits that live in the accumulators.
+template <int ND> struct DzRows {
+    float cg[ND], cb[ND], cl[ND], nls[ND];
+    int lab[ND];
+};
+
+template <int ND>
+__device__ __forceinline__ void dz_rows_init(DzRows<ND>& q, i64 rbase, i64 R, int N, const int2* __restrict__ rowinfo,
+                                             const float2* __restrict__ grads, const float* __restrict__ lse,
+                                             const GradOut go) {
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        const i64 r = rbase + 32 * nd;
+        q.cg[nd] = 0.f; q.cb[nd] = 0.f; q.cl[nd] = 0.f; q.lab[nd] = -1;
+        q.nls[nd] = -INFINITY;  // a row of no usable sequence: 2^-inf * 0 = 0 whatever its logits
+        if (r >= R) continue;
+        const int2 info = rowinfo[r];
+        if (info.y < 0 || info.y >= N) continue;
+        const float g = go.p[(i64)info.y * go.stride] * go.scale;
+        const float2 gr = grads[r];
+        q.lab[nd] = info.x;
+        q.cb[nd] = gr.x * g;
+        q.cl[nd] = info.x >= 0 ? gr.y * g : 0.f;
+        q.cg[nd] = -(gr.x + (info.x >= 0 ? gr.y : 0.f)) * g;
+        q.nls[nd] = -lse[r] * kLog2e;
+    }
+}
+
+template <typename T> struct Pack4;
+template <> struct Pack4<bf16_t> {
+    typedef __bf16 h2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ uint2 of(const float (&o)[4]) {
+        const h2 a = {(__bf16)o[0], (__bf16)o[1]}, b = {(__bf16)o[2], (__bf16)o[3]};
+        return make_uint2(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b));
+    }
+};
+template <> struct Pack4<__half> {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ uint2 of(const float (&o)[4]) {
+        const h2 a = {(_Float16)o[0], (_Float16)o[1]}, b = {(_Float16)o[2], (_Float16)o[3]};
+        return make_uint2(__builtin_bit_cast(unsigned, a), __builtin_bit_cast(unsigned, b));
+    }
+};
+
+// acc[mv][nd] as in fwd_fold_tile; rbase = the lane's data row of nd = 0.  A lane holds runs of four
+// consecutive vocabulary entries of one row.  FAST: the whole tile lies inside the tensor, rows
+// start on 8-byte boundaries (V a multiple of 4) and the blank column is not in this part of the
+// tile: every run leaves as one unguarded 8-byte store.  Otherwise element by element, guarded.
+template <typename T, int NMV, int ND, bool FAST>
+__device__ __forceinline__ void dz_store_tile_as(const f32x16 (&acc)[NMV][ND], int v_first, int V, int blank, int hf,
+                                                 i64 rbase, i64 R, const DzRows<ND>& q, T* __restrict__ dz) {
+    const int bl = blank - v_first;  // same for the whole wave
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        const i64 r = rbase + 32 * nd;
+        // the label's place among the entries of this lane's half, or -1
+        const int lv = q.lab[nd] - v_first - 4 * hf;
+        const int key = (q.lab[nd] >= 0 && lv >= 0 && lv < 32 * NMV && (lv & 4) == 0) ? lv : -1;
+        T* row = dz + r * (i64)V + v_first + 4 * hf;
+#pragma unroll
+        for (int mv = 0; mv < NMV; ++mv)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+                const int e0 = 32 * mv + 8 * b4;  // entry of o[0], relative to v_first + 4 hf
+                float o[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float p = fast_exp2(fmaf(acc[mv][nd][4 * b4 + c], kLog2e, q.nls[nd]));
+                    o[c] = fmaf(p, q.cg[nd], key == e0 + c ? q.cl[nd] : 0.f);
+                }
+                if (FAST) {
+                    *reinterpret_cast<uint2*>(row + e0) = Pack4<T>::of(o);
+                    continue;
+                }
+                if (bl >= e0 && bl < e0 + 8) {  // the blank column lies in this run of one of the two halves
+                    const int cb_at = bl - e0 - 4 * hf;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) o[c] += c == cb_at ? q.cb[nd] : 0.f;
+                }
+                if (r >= R) continue;
+                const int v = v_first + 4 * hf + e0;
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (v + c < V) row[e0 + c] = Elem<T>::from_f32(o[c]);
+            }
+    }
+}
+
+// wave_rows_end: one past the last data row of this wave
+template <typename T, int NMV, int ND>
+__device__ __forceinline__ void dz_store_tile(const f32x16 (&acc)[NMV][ND], int v_first, int V, int blank, int hf,
+                                              i64 rbase, i64 wave_rows_end, i64 R, const DzRows<ND>& q,
+                                              T* __restrict__ dz) {
+    const bool fast = (V & 3) == 0 && v_first + 32 * NMV <= V && wave_rows_end <= R &&
+                      (blank < v_first || blank >= v_first + 32 * NMV);
+    if (fast) dz_store_tile_as<T, NMV, ND, true>(acc, v_first, V, blank, hf, rbase, R, q, dz);
+    else dz_store_tile_as<T, NMV, ND, false>(acc, v_first, V, blank, hf, rbase, R, q, dz);
+}
+
+// ---------------------------------------------------------------------------------------------
+// streaming kernels (any H that is a multiple of 32)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256, 2) void k_joint_fwd(
+    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int H, int V,
+    const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
+    const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
+    int blank, const FwdOut out, int* __restrict__ status) {
+    __shared__ __attribute__((aligned(16))) StreamLds<T> lds;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wd = w & 1, wv = w >> 1;
+    const int hf = lane >> 5, l32 = lane & 31;
+    const i64 row0 = (i64)blockIdx.x * kJM;
+    const i64 rbase = row0 + 128 * wd + l32;  // the rows this lane reduces: rbase + 32 nd, nd = 0..3
+
+    FwdRows<4> q;
+    fwd_rows_init<4>(q, rbase, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
+    walk_streaming<T>(h, W, bias, R, H, V, row0, lds,
+                      [&](const f32x16 (&acc)[2][4], int v_wave) { fwd_fold_tile<2, 4>(acc, v_wave, blank, hf, q); });
+
     // ---- merge: the two halves of a wave, then the two waves that share the data rows ----------
-    float* s_merge = reinterpret_cast<float*>(&s_h[0][0][0]);  // the staging buffers are free now
+    float* s_merge = reinterpret_cast<float*>(&lds.h[0][0][0]);  // the staging buffers are free now
+    fwd_merge_halves<4>(q);
 #pragma unroll
     for (int nd = 0; nd < 4; ++nd) {
-        const float m2 = __shfl_xor(m[nd], 32), s2 = __shfl_xor(s[nd], 32);
-        const float xl2 = __shfl_xor(xl[nd], 32), xb2 = __shfl_xor(xb[nd], 32);
-        lse_merge(m[nd], s[nd], m2, s2);
-        xl[nd] += xl2;  // exactly one of the halves (and of the waves) held the entry, the others 0
-        xb[nd] += xb2;
         if (wv == 1 && hf == 0) {
-            float* q = s_merge + ((wd * 4 + nd) * 32 + l32) * 4;
-            q[0] = m[nd]; q[1] = s[nd]; q[2] = xl[nd]; q[3] = xb[nd];
+            float* p = s_merge + ((wd * 4 + nd) * 32 + l32) * 4;
+            p[0] = q.m[nd]; p[1] = q.s[nd]; p[2] = q.xl[nd]; p[3] = q.xb[nd];
         }
     }
     __syncthreads();
     if (wv != 0 || hf != 0) return;
 #pragma unroll
     for (int nd = 0; nd < 4; ++nd) {
-        const i64 r = row0 + 128 * wd + 32 * nd + l32;
+        const i64 r = rbase + 32 * nd;
         if (r >= R) continue;
-        const float* q = s_merge + ((wd * 4 + nd) * 32 + l32) * 4;
-        lse_merge(m[nd], s[nd], q[0], q[1]);
-        const Lse lse = {m[nd], log2_of_sum(s[nd])};
-        lse_out[r] = lse.value();
-        const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-        rowinfo[r] = make_int2(lab[nd] < 0 ? -1 : lab[nd], ri.n);
-        if (pad >= 0)
-            lp[pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1)] =
-                make_lp(xb[nd] + q[3], xl[nd] + q[2], lse, lab[nd], seqmode + ri.n);
-        else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
+        const float* p = s_merge + ((wd * 4 + nd) * 32 + l32) * 4;
+        lse_merge(q.m[nd], q.s[nd], p[0], p[1]);
+        fwd_row_out(r, R, q.m[nd], q.s[nd], q.xb[nd] + p[3], q.xl[nd] + p[2], q.lab[nd], lx, ly, row_off, pad_off, N,
+                    out);
     }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256, 2) void k_joint_dz(
+    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int H, int V, int N,
+    int blank, const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
+    const GradOut go, T* __restrict__ dz) {
+    __shared__ __attribute__((aligned(16))) StreamLds<T> lds;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wd = w & 1;
+    const int hf = lane >> 5, l32 = lane & 31;
+    const i64 row0 = (i64)blockIdx.x * kJM;
+    const i64 rbase = row0 + 128 * wd + l32;
+    DzRows<4> q;
+    dz_rows_init<4>(q, rbase, R, N, rowinfo, grads, lse, go);
+    walk_streaming<T>(h, W, bias, R, H, V, row0, lds, [&](const f32x16 (&acc)[2][4], int v_wave) {
+        dz_store_tile<T, 2, 4>(acc, v_wave, V, blank, hf, rbase, row0 + 128 * wd + 128, R, q, dz);
+    });
+}
+
 // ---------------------------------------------------------------------------------------------
-// forward, data rows resident in registers
+// data rows resident in registers
 // ---------------------------------------------------------------------------------------------
-// The streaming kernel above reads its h tile once per vocabulary tile: V / 128 times in all, from
+// The streaming kernels above read their h tile once per vocabulary tile: V / 128 times in all, from
 // HBM, since the tiles of all resident workgroups together exceed the L2 (measured on N=32, V=1024,
 // H=512: 3.3 GB fetched for 0.32 GB of h, and the kernel runs at the speed of that traffic).  Here
 // every wave keeps the MFMA operand fragments of its OWN 32 ND data rows in registers for the whole
@@ -281,46 +477,40 @@ __global__ __launch_bounds__(256, 2) void k_joint_fwd(
 constexpr int kRK = 64;      // K-slice of the weight tile
 constexpr int kRPitch = 72;  // 144 bytes: 16 consecutive rows start in 16 different groups of four banks
 
-template <typename T, int ND, int KS /* H / 16 */, int OCC, bool D2>
-__global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
-    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
-    const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
-    const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
-    int blank, LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
-    float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
-    constexpr int H = KS * 16;
-    constexpr int NK = H / kRK;  // K-slices per vocabulary tile
-    static_assert(H % kRK == 0, "whole K-slices");
-    __shared__ __attribute__((aligned(16))) T s_w[2][kJN][kRPitch];
-    __shared__ __attribute__((aligned(16))) float s_bias[2][kJN];  // what the accumulators of a tile start from
+template <typename T> struct ResLds {
+    T w[2][kJN][kRPitch];
+    float bias[2][kJN];  // what the accumulators of a tile start from
+};
 
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+// this wave's data rows [row0, row0 + 32 ND), as MFMA operand fragments
+template <typename T, int ND, int KS /* H / 16 */>
+__device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 R, i64 row0, v4i (&hreg)[ND][KS]) {
+    const int lane = threadIdx.x & 63;
     const int hf = lane >> 5, l32 = lane & 31;
-    const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);  // first data row of this wave
     const i64 last_row = R - 1;
-
-    // ---- this wave's data rows, as MFMA operand fragments, for good ----------
-    v4i hreg[ND][KS];
 #pragma unroll
     for (int nd = 0; nd < ND; ++nd) {
         i64 r = row0 + 32 * nd + l32;
         r = r < last_row ? r : last_row;  // rows beyond the tensor are multiplied like the last one and dropped
-        const T* src = h + r * (i64)H + 8 * hf;
+        const T* src = h + r * (i64)(KS * 16) + 8 * hf;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) hreg[nd][ks] = *reinterpret_cast<const v4i*>(src + 16 * ks);
     }
-    int lab[ND];
-#pragma unroll
-    for (int nd = 0; nd < ND; ++nd) {
-        const i64 r = row0 + 32 * nd + l32;
-        lab[nd] = kNoLabel;
-        if (r < R) {
-            const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-            if (ri.n >= 0 && pad_off[ri.n] >= 0) lab[nd] = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
-        }
-    }
+}
+
+// tile(acc, v0) receives acc[mv][nd] = vocabulary entries [v0 + 32 mv, v0 + 32 mv + 32) x data rows
+// [32 nd, 32 nd + 32) of the wave's rows in hreg
+template <typename T, int ND, int KS, bool D2, typename TileFn>
+__device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T* __restrict__ W,
+                                              const float* __restrict__ bias, int V, ResLds<T>& lds, TileFn&& tile) {
+    constexpr int H = KS * 16;
+    constexpr int NK = H / kRK;  // K-slices per vocabulary tile
+    static_assert(H % kRK == 0, "whole K-slices");
+    auto& s_w = lds.w;
+    auto& s_bias = lds.bias;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int hf = lane >> 5, l32 = lane & 31;
 
     // ---- weight tile: thread t moves 16-byte piece (t % 8) of rows t / 8 + 32 p, p = 0..3 ----------
     const int st_row = tid >> 3, st_piece = tid & 7;
@@ -340,10 +530,6 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
         for (int p = 0; p < 4; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + 32 * p][st_piece * 8]) = q.w[p];
     };
 
-    float m[ND], s[ND], xl[ND], xb[ND];
-#pragma unroll
-    for (int nd = 0; nd < ND; ++nd) { m[nd] = -INFINITY; s[nd] = 0.f; xl[nd] = 0.f; xb[nd] = 0.f; }
-
     // slices are numbered it = vt * NK + kc; slice it is multiplied out of buffer it & 1 (NK is even
     // or the parity is carried), its loads were issued two slices earlier
     // the bias of a tile (-inf beyond the vocabulary, which no finite product changes and which drops
@@ -362,7 +548,6 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     f32x16 acc[4][ND];
     int par = 0;  // buffer of the current slice
     for (int vt = 0; vt < nvt; ++vt) {
-        const int v0 = vt * kJN;
 #pragma unroll
         for (int mv = 0; mv < 4; ++mv)
 #pragma unroll
@@ -413,91 +598,83 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
             __syncthreads();
             par ^= 1;
         }
-
-        // ---- fold the tile's logits into the rows' running state ----------
-        const int blank_key = (blank >= v0 && blank < v0 + kJN && (((blank - v0) >> 2) & 1) == hf) ? blank - v0 : -1;
-#pragma unroll
-        for (int nd = 0; nd < ND; ++nd) {
-            float mx = acc[0][nd][0];
-#pragma unroll
-            for (int mv = 0; mv < 4; ++mv)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc[mv][nd][r]);
-            const float mn = fmaxf(m[nd], mx);
-            if (mn > -INFINITY) {
-                const float ms = mn * kLog2e;
-                float sum = s[nd] * fast_exp2(fmaf(m[nd], kLog2e, -ms));  // m = -inf: s = 0 stays 0
-#pragma unroll
-                for (int mv = 0; mv < 4; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sum += fast_exp2(fmaf(acc[mv][nd][r], kLog2e, -ms));
-                s[nd] = sum;
-                m[nd] = mn;
-            }
-            const int lv = lab[nd] - v0;
-            const int key = (lab[nd] >= 0 && lv >= 0 && lv < kJN && ((lv >> 2) & 1) == hf) ? lv : -1;
-            if (__ballot(key >= 0) != 0) {
-#pragma unroll
-                for (int mv = 0; mv < 4; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) xl[nd] = key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : xl[nd];
-            }
-            if (__ballot(blank_key >= 0) != 0) {
-#pragma unroll
-                for (int mv = 0; mv < 4; ++mv)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        xb[nd] = blank_key == 32 * mv + acc_row(r, hf) ? acc[mv][nd][r] : xb[nd];
-            }
-        }
-    }
-
-    // ---- the two halves of the wave hold disjoint vocabulary entries of the same rows ----------
-#pragma unroll
-    for (int nd = 0; nd < ND; ++nd) {
-        lse_merge(m[nd], s[nd], __shfl_xor(m[nd], 32), __shfl_xor(s[nd], 32));
-        xl[nd] += __shfl_xor(xl[nd], 32);  // exactly one half held the entry, the other 0
-        xb[nd] += __shfl_xor(xb[nd], 32);
-        const i64 r = row0 + 32 * nd + l32;
-        if (hf != 0 || r >= R) continue;
-        const Lse lse = {m[nd], log2_of_sum(s[nd])};
-        lse_out[r] = lse.value();
-        const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
-        const i64 pad = ri.n >= 0 ? pad_off[ri.n] : -1;
-        rowinfo[r] = make_int2(lab[nd] < 0 ? -1 : lab[nd], ri.n);
-        if (pad >= 0)
-            lp[pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1)] = make_lp(xb[nd], xl[nd], lse, lab[nd], seqmode + ri.n);
-        else if (grads_skipped) grads_skipped[r] = make_float2(0.f, 0.f);
+        tile(acc, vt * kJN);
     }
 }
+
+template <typename T, int ND, int KS, int OCC, bool D2>
+__global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
+    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
+    const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
+    const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
+    int blank, const FwdOut out, int* __restrict__ status) {
+    __shared__ __attribute__((aligned(16))) ResLds<T> lds;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int hf = lane >> 5, l32 = lane & 31;
+    const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);  // first data row of this wave
+    v4i hreg[ND][KS];
+    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
+    FwdRows<ND> q;
+    fwd_rows_init<ND>(q, row0 + l32, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
+    walk_resident<T, ND, KS, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[4][ND], int v0) {
+        fwd_fold_tile<4, ND>(acc, v0, blank, hf, q);
+    });
+    fwd_merge_halves<ND>(q);
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        const i64 r = row0 + 32 * nd + l32;
+        if (hf != 0 || r >= R) continue;
+        fwd_row_out(r, R, q.m[nd], q.s[nd], q.xb[nd], q.xl[nd], q.lab[nd], lx, ly, row_off, pad_off, N, out);
+    }
+}
+
+template <typename T, int ND, int KS, int OCC, bool D2>
+__global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
+    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V, int N, int blank,
+    const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
+    const GradOut go, T* __restrict__ dz) {
+    __shared__ __attribute__((aligned(16))) ResLds<T> lds;
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int hf = lane >> 5, l32 = lane & 31;
+    const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);
+    v4i hreg[ND][KS];
+    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
+    DzRows<ND> q;
+    dz_rows_init<ND>(q, row0 + l32, R, N, rowinfo, grads, lse, go);
+    walk_resident<T, ND, KS, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[4][ND], int v0) {
+        dz_store_tile<T, 4, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz);
+    });
+}
+
+// The joint sizes in use take the resident kernels; any other multiple of 32 the streaming ones.
+// Measured on R = 311449, V = 1024, H = 512 (bf16): one data block per wave at two waves per SIMD
+// 0.46 ms; two blocks per wave at one wave per SIMD 0.63 ms (registers spill); streaming kernel 0.63 ms.
+#define CWR_JOINT_SHAPES(X) X(2, 16, 1, true) X(2, 24, 1, true) X(1, 32, 2, false) X(1, 40, 1, true) \
+                            X(1, 48, 1, true) X(1, 64, 1, true)
 
 template <typename T>
 static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
                               float* grads) {
-    int2* ri = reinterpret_cast<int2*>(rowinfo);
-    float2* gz = reinterpret_cast<float2*>(grads);
+    const FwdOut out = {ws.lp, lse, reinterpret_cast<int2*>(rowinfo), reinterpret_cast<float2*>(grads), ws.seqmode};
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
-#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                              \
-    if (j.H == 16 * KS) {                                                                                       \
-        const i64 blocks = (b.R + 128 * ND - 1) / (128 * ND);                                                   \
-        if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                    \
-        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w, j.bias,  \
-                   b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N,       \
-                   b.blank, ws.lp, lse, ri, gz, ws.seqmode, b.status);                                          \
-        return check_launch();                                                                                  \
+#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                           \
+    if (j.H == 16 * KS) {                                                                                        \
+        const i64 blocks = (b.R + 128 * ND - 1) / (128 * ND);                                                    \
+        if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                     \
+        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w,  \
+                   j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,     \
+                   b.N, b.blank, out, b.status);                                                                 \
+        return check_launch();                                                                                   \
     }
-    // the joint sizes in use; any other multiple of 32 takes the streaming kernel
-    // measured on R = 311449, V = 1024, H = 512 (bf16): one data block per wave at two waves per SIMD
-    // 0.46 ms; two blocks per wave at one wave per SIMD 0.63 ms (registers spill); streaming kernel 0.63 ms
-    CWR_JOINT_RES(2, 16, 1, true) CWR_JOINT_RES(2, 24, 1, true) CWR_JOINT_RES(1, 32, 2, false)
-    CWR_JOINT_RES(1, 40, 1, true) CWR_JOINT_RES(1, 48, 1, true) CWR_JOINT_RES(1, 64, 1, true)
+    CWR_JOINT_SHAPES(CWR_JOINT_RES)
 #undef CWR_JOINT_RES
     const i64 blocks = (b.R + kJM - 1) / kJM;
     if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
     CWR_LAUNCH((k_joint_fwd<T>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w, j.bias, b.R, (int)j.H, b.V,
-               b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, ws.lp, lse, ri, gz,
-               ws.seqmode, b.status);
+               b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, out, b.status);
     return check_launch();
 }
 
@@ -506,6 +683,42 @@ int launch_joint_gather(const Batch& b, const Workspace& ws, const JointOperands
     if (b.R == 0) return CWR_OK;
     if (b.dtype == CWR_BF16) return joint_gather_typed<bf16_t>(b, ws, j, lse, rowinfo, grads);
     if (b.dtype == CWR_F16) return joint_gather_typed<__half>(b, ws, j, lse, rowinfo, grads);
+    return CWR_ERR_DTYPE;
+}
+
+template <typename T>
+static int joint_dlogits_typed(const JointOperands& j, i64 R, int V, int N, int blank, const int* rowinfo,
+                               const float* grads, const float* lse, const GradOut go, void* dlogits,
+                               hipStream_t stream) {
+    const int2* ri = reinterpret_cast<const int2*>(rowinfo);
+    const float2* gr = reinterpret_cast<const float2*>(grads);
+    const T* h = static_cast<const T*>(j.h);
+    const T* w = static_cast<const T*>(j.w);
+    T* dz = static_cast<T*>(dlogits);
+#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                          \
+    if (j.H == 16 * KS) {                                                                                       \
+        const i64 blocks = (R + 128 * ND - 1) / (128 * ND);                                                     \
+        if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                    \
+        CWR_LAUNCH((k_joint_dz_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, stream, h, w,    \
+                   j.bias, R, V, N, blank, ri, gr, lse, go, dz);                                                \
+        return check_launch();                                                                                  \
+    }
+    CWR_JOINT_SHAPES(CWR_JOINT_RES)
+#undef CWR_JOINT_RES
+    const i64 blocks = (R + kJM - 1) / kJM;
+    if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
+    CWR_LAUNCH((k_joint_dz<T>), dim3((unsigned)blocks), dim3(256), 0, stream, h, w, j.bias, R, (int)j.H, V, N, blank,
+               ri, gr, lse, go, dz);
+    return check_launch();
+}
+
+int launch_joint_dlogits(int dtype, const JointOperands& j, i64 R, i64 V, i64 N, int blank, const int* rowinfo,
+                         const float* grads, const float* lse, const GradOut go, void* dlogits, hipStream_t stream) {
+    if (R == 0) return CWR_OK;
+    if (dtype == CWR_BF16)
+        return joint_dlogits_typed<bf16_t>(j, R, (int)V, (int)N, blank, rowinfo, grads, lse, go, dlogits, stream);
+    if (dtype == CWR_F16)
+        return joint_dlogits_typed<__half>(j, R, (int)V, (int)N, blank, rowinfo, grads, lse, go, dlogits, stream);
     return CWR_ERR_DTYPE;
 }
 

@@ -11,9 +11,10 @@ from typing import Any, Optional
 import torch
 
 from . import _lib
-from .loss import _DTYPES, _offsets, _raise_on_status, _stream_ptr
+from .loss import _DTYPES, _offsets, _raise_on_flags, _raise_on_status, _stream_ptr, joint_forward
 
 _ACTS = {None: 0, "none": 0, "tanh": 1, "relu": 2}
+_DW_SPLIT = 16  # parts the rows of a block are cut into for the weight-gradient product
 
 
 class _Join(torch.autograd.Function):
@@ -83,6 +84,94 @@ def compact_join(f: torch.Tensor, g: torch.Tensor, lx: torch.Tensor, ly: torch.T
     return out
 
 
+class _JointLoss(torch.autograd.Function):
+    """Loss of logits = h @ weight.T + bias that are never stored.
+
+    Forward: cwr_joint_forward (the output layer on the matrix cores, every tile reduced on the spot
+    to the row's log-sum-exp and its blank / label logits).  Backward: cwr_joint_backward forms the
+    logits of a block of rows again on the matrix cores and writes their gradient, rounded once to
+    the 16-bit type; library GEMMs multiply the block into dh, dW and dbias.  Only
+    `chunk_rows` x V logit gradients exist at any moment."""
+
+    @staticmethod
+    def forward(ctx: Any, h, weight, bias, lx, ys, ly, blank, reduction, max_u, validate, chunk_rows):
+        costs, st = joint_forward(h, weight, bias, lx, ys, ly, blank, max_u)
+        if validate:
+            _raise_on_flags(st)
+        st.workspace = None
+        ctx.state = st
+        ctx.blank, ctx.reduction, ctx.chunk_rows = blank, reduction, int(chunk_rows)
+        ctx.save_for_backward(h, weight, bias if bias is not None else h.new_empty(0), lx, ys, ly)
+        ctx.has_bias = bias is not None
+        if reduction == "mean":
+            return costs.mean()
+        if reduction == "sum":
+            return costs.sum()
+        return costs
+
+    @staticmethod
+    def backward(ctx: Any, grad_out):
+        h, weight, bias, lx, ys, ly = ctx.saved_tensors
+        st = ctx.state
+        lib = _lib.load()
+        dev = h.device
+        R, H = h.shape
+        V = weight.size(0)
+        N = st.N
+        gc = grad_out.to(torch.float32).reshape(-1)
+        if gc.numel() == 1:
+            gc = gc.expand(N)
+        gc = (gc / N if ctx.reduction == "mean" else gc).contiguous()
+        dh = torch.empty_like(h)
+        dw = torch.zeros((V, H), dtype=torch.float32, device=dev)
+        db = torch.zeros(V, dtype=torch.float32, device=dev) if ctx.has_bias else None
+        bias_f = bias.to(torch.float32).contiguous() if ctx.has_bias else None
+        chunk = max(1, min(ctx.chunk_rows, R))
+        z = torch.empty((chunk, V), dtype=h.dtype, device=dev)
+        with torch.cuda.device(dev):
+            stream = _stream_ptr(dev)
+            for r0 in range(0, R, chunk):
+                r1 = min(R, r0 + chunk)
+                zc = z[: r1 - r0]
+                rc = lib.cwr_joint_backward(h[r0:].data_ptr(), weight.data_ptr(),
+                                            bias_f.data_ptr() if bias_f is not None else None, _DTYPES[h.dtype],
+                                            r1 - r0, H, V, N, int(ctx.blank), st.rowinfo[r0:].data_ptr(),
+                                            st.grads[r0:].data_ptr(), st.lse[r0:].data_ptr(), gc.data_ptr(), 1, 1.0,
+                                            zc.data_ptr(), stream)
+                _lib.check(rc, "cwr_joint_backward")
+                torch.mm(zc, weight, out=dh[r0:r1])
+                # dW += zc^T h[r0:r1].  The contraction runs over the rows, the result is only (V, H): as one
+                # GEMM the library fills a quarter of the GPU with it, so the rows are cut into _DW_SPLIT
+                # parts multiplied as a batch (16-bit products of a part each, summed in fp32)
+                n = r1 - r0
+                m = (n // _DW_SPLIT) * _DW_SPLIT
+                if m:
+                    part = torch.bmm(zc[:m].view(_DW_SPLIT, m // _DW_SPLIT, V).transpose(1, 2),
+                                     h[r0:r0 + m].view(_DW_SPLIT, m // _DW_SPLIT, H))
+                    dw.add_(part.sum(dim=0, dtype=torch.float32))
+                if n > m:
+                    dw.add_(torch.mm(zc[m:n].t(), h[r0 + m:r1]))
+                if db is not None:
+                    db.add_(zc.sum(dim=0, dtype=torch.float32))
+        dbias = db.to(bias.dtype) if db is not None else None
+        return dh, dw.to(weight.dtype), dbias, None, None, None, None, None, None, None, None
+
+
+def fused_joint_loss(h: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], lx: torch.Tensor,
+                     y: torch.Tensor, ly: torch.Tensor, blank: int = 0, reduction: Optional[str] = "mean", *,
+                     max_u: Optional[int] = None, validate: bool = False, chunk_rows: int = 131072) -> torch.Tensor:
+    """transducer_loss(h @ weight.T + bias, lx, y, ly, blank, reduction, fused_log_softmax=True) without
+    the (R, V) logits: h (R, H) compact joint activations (e.g. from compact_join), weight (V, H) and
+    bias (V,) or None the output layer, fp16 or bf16.  Differentiable in h, weight and bias; the
+    backward pass holds at most chunk_rows x V logits at a time."""
+    assert lx.dtype == torch.int32 and ly.dtype == torch.int32 and y.dtype == torch.int32
+    assert reduction in ["mean", "sum", "none"] or reduction is None
+    assert blank >= 0 and blank < weight.size(0)
+    return _JointLoss.apply(h.contiguous(), weight.contiguous(), bias, lx, y, ly, int(blank),
+                            reduction if reduction in ("mean", "sum") else "none", max_u, bool(validate),
+                            int(chunk_rows))
+
+
 class CompactJoiner(torch.nn.Module):
     """Projection of encoder and predictor outputs to a joint space, their compact broadcast sum
     with an activation, and the output layer: (N,T,E), (N,U+1,P) -> (R, V) logits in the layout
@@ -99,3 +188,10 @@ class CompactJoiner(torch.nn.Module):
     def forward(self, enc_out, pred_out, lx, ly, total_rows: Optional[int] = None):
         h = compact_join(self.enc(enc_out), self.pred(pred_out), lx, ly, self.activation, total_rows)
         return self.out(h)
+
+    def loss(self, enc_out, pred_out, lx, y, ly, blank: int = 0, reduction: Optional[str] = "mean",
+             total_rows: Optional[int] = None):
+        """The transducer loss of this joiner's logits without storing them (fp16 / bf16 modules):
+        compact_join, then fused_joint_loss on the output layer's weight and bias."""
+        h = compact_join(self.enc(enc_out), self.pred(pred_out), lx, ly, self.activation, total_rows)
+        return fused_joint_loss(h, self.out.weight, self.out.bias, lx, y, ly, blank, reduction)

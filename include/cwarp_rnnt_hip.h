@@ -294,6 +294,21 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
                       int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
                       float* grads, float* costs, void* stream);
 
+/* Backward of cwr_joint_forward, one block of rows at a time: the logits of rows [0, R) of the block
+ * are formed again on the matrix cores (fp32 accumulators) and turned in registers into
+ *   dlogits[r, v] = g * (softmax(logits_r)[v] * gamma_r + grads[r,0] [v == blank] + grads[r,1] [v == label]),
+ * cwr_backward's CWR_MODE_FUSED formula (cwarp_cuda_rnnt_kernel.cu:518-519 and
+ * cwarp_cuda_gather_kernel.cu:52-74 behind a log-softmax), rounded once to `dtype` and written to
+ * dlogits (R, V).  The caller multiplies the block into dh = dlogits w, dW += dlogits^T h,
+ * dbias += column sums (plain GEMMs) and reuses the buffer for the next block, so that at most one
+ * block of logit gradients exists at a time.  The reference repository has no joiner.
+ *   h, rowinfo, grads, lse, dlogits  point at the block's first row;  rowinfo, grads, lse as
+ *   written by cwr_joint_forward;  w, bias, dtype, H, V, N, blank as there;
+ *   grad_costs, grad_stride, grad_scale as for cwr_backward. */
+int cwr_joint_backward(const void* h, const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                       int64_t N, int32_t blank, const int32_t* rowinfo, const float* grads, const float* lse,
+                       const float* grad_costs, int64_t grad_stride, float grad_scale, void* dlogits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

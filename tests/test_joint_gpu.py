@@ -62,3 +62,88 @@ def test_joint_forward_matches_oracle(dtype, lx, ly, H, V, bias):
         want_lab = np.tile(np.concatenate([j["yp"][n, :U], [-1]]), T)
         assert np.array_equal(ri[off[n]:off[n + 1], 0], want_lab)
         assert np.all(ri[off[n]:off[n + 1], 1] == n)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("lx,ly,H,V,bias,blank", [
+    ([9, 5, 12, 1], [3, 0, 7, 4], 64, 128, True, 0),
+    ([40, 33, 17], [12, 20, 5], 96, 300, True, 299),      # ragged last tile; the blank in it (streaming kernel)
+    ([50, 21], [30, 70], 256, 1024, False, 77),           # resident kernel, two data blocks per wave
+    ([50, 21], [30, 20], 512, 515, True, 130),            # resident kernel; V not a multiple of 4: element stores
+    ([30, 14], [9, 3], 32, 40, True, 5),
+])
+def test_joint_backward_dlogits_match_oracle(dtype, lx, ly, H, V, bias, blank):
+    """cwr_joint_backward through the C ABI, a block of rows at a time (blocks that end inside a
+    kernel's group of rows), against the oracle's dense fused gradient of the float64 logits.
+    Tolerance: the one rounding of the result to the 16-bit type (2^-8 / 2^-11 relative) plus the
+    fp32 evaluation of softmax (1e-5 of the row's largest entry)."""
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd import _lib
+    from compactwarprnntloss_amd.loss import _DTYPES, _stream_ptr
+    j = make_joint(lx, ly, H, V, seed=4, dtype=dtype, scale=3.0, bias=bias)
+    N, R = j["N"], j["R"]
+    go = np.random.default_rng(2).uniform(0.5, 1.5, N)
+    z = orc.joint_logits(j["h"].double().numpy(), j["w"].double().numpy(), None if j["b"] is None else j["b"].numpy())
+    ref = orc.loss_and_grad(z, j["lx"], j["yp"], j["ly"], blank, "fused", grad_out=go, want_dense=True)
+    h, W = j["h"].to(DEV), j["w"].to(DEV)
+    b = None if j["b"] is None else j["b"].to(DEV)
+    costs, st = pkg.joint_forward(h, W, b, torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["yp"]).to(DEV),
+                                  torch.from_numpy(j["ly"]).to(DEV), blank)
+    gc = torch.from_numpy(go).float().to(DEV)
+    dz = torch.full((R, V), float("nan"), dtype=TDT[dtype], device=DEV)
+    lib = _lib.load()
+    block = 173
+    for r0 in range(0, R, block):
+        n = min(block, R - r0)
+        rc = lib.cwr_joint_backward(h[r0:].data_ptr(), W.data_ptr(), b.data_ptr() if b is not None else None,
+                                    _DTYPES[TDT[dtype]], n, H, V, N, blank, st.rowinfo[r0:].data_ptr(),
+                                    st.grads[r0:].data_ptr(), st.lse[r0:].data_ptr(), gc.data_ptr(), 1, 1.0,
+                                    dz[r0:].data_ptr(), _stream_ptr(torch.device(DEV)))
+        assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    got = dz.double().cpu().numpy()
+    eps = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    tol = eps * np.abs(ref["grad"]) + 2e-5 * np.abs(ref["grad"]).max(axis=1, keepdims=True) + 1e-7
+    assert np.all(np.isfinite(got))
+    bad = np.abs(got - ref["grad"]) > tol
+    assert not bad.any(), (np.argwhere(bad)[:5], got[bad][:5], ref["grad"][bad][:5])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("reduction", ["mean", "none"])
+def test_fused_joint_loss_gradients_match_oracle(dtype, reduction):
+    """loss -> (dh, dW, dbias) through the autograd node, against the oracle's chain rule
+    (dense fused gradient of the float64 logits, then joint_backward).  The backward pass forms the
+    logits a block of rows at a time; a small block size makes the test cross several blocks.
+    Tolerance of the gradients: one rounding of d logits to the 16-bit type before the products."""
+    import compactwarprnntloss_amd as pkg
+    j = make_joint([40, 33, 17], [12, 20, 5], 96, 300 if dtype == "bf16" else 256, seed=9, dtype=dtype, scale=3.0)
+    N = j["N"]
+    w = np.random.default_rng(1).uniform(0.5, 1.5, N)
+    go = w / N if reduction == "mean" else w
+    z, ref = reference(j, grad_out=go, want_dense=True)
+    dh_ref, dw_ref, db_ref = orc.joint_backward(ref["grad"], j["h"].double().numpy(), j["w"].double().numpy())
+    h = j["h"].to(DEV).requires_grad_(True)
+    W = j["w"].to(DEV).requires_grad_(True)
+    b = j["b"].to(DEV).requires_grad_(True)
+    lx, ly = torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV)
+    y = torch.from_numpy(j["yp"]).to(DEV)
+    wt = torch.from_numpy(w).to(DEV).float()
+    if reduction == "mean":
+        # per-sequence weights through a mean: weight the costs by hand
+        costs = pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "none", chunk_rows=257)
+        loss = (costs * wt).mean()
+    else:
+        loss = (pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "none", chunk_rows=257) * wt).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    rel = 1e-2 if dtype == "bf16" else 2e-3
+    for got, want, name in ((h.grad, dh_ref, "dh"), (W.grad, dw_ref, "dW"), (b.grad, db_ref, "dbias")):
+        got = got.double().cpu().numpy()
+        scale = np.abs(want).max()
+        np.testing.assert_allclose(got, want, rtol=rel, atol=rel * scale, err_msg=name)
+    # and the value itself, with the reduction done by the node
+    with torch.no_grad():
+        lm = pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "mean")
+    _, ref1 = reference(j)
+    assert abs(float(lm) - ref1["costs"].mean()) <= LOSS_RTOL * ref1["costs"].mean()

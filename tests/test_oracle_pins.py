@@ -343,3 +343,35 @@ def test_row_lse_matches_scipy_for_every_storage_type():
         x = (rng.standard_normal((5000, 37)) * 6).astype(dt)
         x[17] = 30000 if dt == np.float16 else 1e4   # exp would overflow without the row maximum
         np.testing.assert_allclose(orc.row_lse(x, chunk=999), logsumexp(x.astype(np.float64), axis=-1), rtol=1e-14)
+
+
+def test_joint_layer_restatement_against_finite_differences_and_torch():
+    """joint_logits / joint_backward (no reference counterpart): the matrix product against torch in
+    float64, the backward against central finite differences of the loss of those logits."""
+    import torch
+    rng = np.random.default_rng(5)
+    lx, ly = np.array([3, 2], np.int32), np.array([2, 1], np.int32)
+    R, H, V = int(orc.row_offsets_i64(lx, ly)[-1]), 5, 7
+    h, w, b = rng.standard_normal((R, H)), rng.standard_normal((V, H)), rng.standard_normal(V)
+    y = np.array([[1, 3], [2, 0]], np.int32)
+    z = orc.joint_logits(h, w, b)
+    zt = torch.from_numpy(h) @ torch.from_numpy(w).T + torch.from_numpy(b)
+    np.testing.assert_allclose(z, zt.numpy(), rtol=1e-13, atol=1e-13)
+    ref = orc.loss_and_grad(z, lx, y, ly, 0, "fused")
+    dh, dw, db = orc.joint_backward(ref["grad"], h, w)
+
+    def total(hh, ww, bb):
+        return orc.loss_and_grad(orc.joint_logits(hh, ww, bb), lx, y, ly, 0, "fused", want_dense=False)["costs"].sum()
+
+    eps = 1e-6
+    for arr, grad in ((h, dh), (w, dw), (b, db)):
+        it = np.nditer(arr, flags=["multi_index"])
+        for _ in it:
+            idx = it.multi_index
+            keep = arr[idx]
+            arr[idx] = keep + eps
+            up = total(h, w, b)
+            arr[idx] = keep - eps
+            dn = total(h, w, b)
+            arr[idx] = keep
+            assert abs((up - dn) / (2 * eps) - grad[idx]) < 1e-6, (idx, (up - dn) / (2 * eps), grad[idx])
