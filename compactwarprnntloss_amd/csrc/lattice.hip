@@ -213,7 +213,11 @@ struct Ring {
 
 // What a wait needs besides its counter: where to report, the workgroup's abort word, and how many
 // polls to spend.  A wait that runs out sets the abort word; every later wait of the workgroup sees
-// it first and returns at once, so a broken hand-over costs ONE spin budget, not one per block.
+// it first and returns at once, so a broken hand-over costs ONE spin budget, not one per block.  The
+// walks do not leave their loops on a failed wait (an extra way out of the block loop makes the
+// register allocator rotate the prefetch ring through copies, +15 % per block): they run on at
+// their normal pace over values nobody will use, every access still inside its buffer, and the
+// workgroup marks the sequence as poisoned at the end.
 struct WaitCtl {
     int* status;  // the call's status word (global)
     int* abort;   // LDS, one per workgroup
@@ -323,7 +327,6 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
     const int p16 = nl * 16, p8 = nl * 8, p4 = nl * 4;
-    bool gave_up = false;
     const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * p4);
@@ -384,15 +387,14 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
                 cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
             }
             if (HAS_IN && prod < k0 + kPF + in_shift) {
-                gave_up = !wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
+                wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
                 keep_order();
                 en_first = rin.slots[(k0 + jl + in_shift) & (kRing - 1)];
                 cp_first = rin.scales[((k0 + jl + in_shift) / kPF) & (kRing / kPF - 1)];
             }
             if (HAS_OUT && cons < k0 + kPF - kRing - out_shift)
-                gave_up = !wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc) || gave_up;
+                wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc);
         }
-        if ((HAS_IN || HAS_OUT) && gave_up) break;  // wave-uniform: the counters are
         keep_order();
         // Renew the scales.  True magnitude (binary exponent minus scale) of what the lane holds,
         // of what it will hand over and of what its neighbour will hand over next:
@@ -490,10 +492,6 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         if (HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    if (gave_up) {  // nobody is to wait for this strip any more
-        if (HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
     return __ballot(lo_seen < kLowHigh - 1u || hi_seen >= kHighHigh) == 0;
 }
 
@@ -507,7 +505,6 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
                                                 double* out_strip, const double* bnd_in, double* bnd_out,
                                                 const Ring rin, const Ring rout, const WaitCtl wc) {
     const int lane = threadIdx.x & 63;
-    bool gave_up = false;
     const int Q = T + nl - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
@@ -554,9 +551,8 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
         // entries [k0+in_shift, k0+kPF+in_shift) must have been produced; the ring slots of entries
         // [k0, k0+kPF) must be free, i.e. the consumer (which reads entry i at its step
         // i-out_shift) must be past entry k0+kPF-1-kRing
-        if (CONC && HAS_IN) gave_up = !wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
-        if (CONC && HAS_OUT) gave_up = !wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc) || gave_up;
-        if (CONC && gave_up) break;
+        if (CONC && HAS_IN) wait_at_least(rin.produced, k0 + kPF + in_shift, wc);
+        if (CONC && HAS_OUT) wait_at_least(rout.consumed, k0 + kPF - kRing - out_shift, wc);
         if (CONC) keep_order();
         double e_lane = kNeg;
         if (HAS_IN) {
@@ -605,10 +601,6 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
         const int done = blk + 1 == nblocks ? 0x7fffffff : k0 + kPF;
         if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-    if (CONC && gave_up) {
-        if (HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
 }
 
