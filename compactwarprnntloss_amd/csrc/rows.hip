@@ -393,6 +393,13 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         my_dst = pad + lattice_slot(ri.t, ri.u, ri.T, (i64)ri.U + 1);
     }
 
+    // The two entries the loss wants of each row are picked out of LDS: every pass parks its packs
+    // there as loaded (a wave's LDS accesses are served in order, so no barrier is needed for its
+    // own region) and each lane reads its row's blank and label entry back.  Picking them out of
+    // the registers instead takes a chain of selects and cross-lane reads per row, which is what
+    // this kernel, bound by its vector instructions on rows this short, can least afford.
+    __shared__ __attribute__((aligned(16))) v4i s_stage[kWavesPerBlock][RP * (LPR * K + 1)];
+    v4i* stage = s_stage[__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))] + g * (LPR * K + 1);
     const ColPos<VEC, LPR> pb(blank);
     Lse res_lse = {0.f, 0.f};
     float res_b = 0.f, res_l = 0.f;  // results of the lane's own row
@@ -402,6 +409,8 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
 #pragma unroll
         for (int k = 0; k < K; ++k)
             if (!(ok && lir + k * LPR < NV)) raw[p][k] = Pack<T>::neg_inf();
+#pragma unroll
+        for (int k = 0; k < K; ++k) stage[lir + k * LPR] = raw[p][k];
         // the label of the row of this pass, from the lane that decoded it
         int lab;
         if (RP <= 2) {
@@ -410,9 +419,12 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
         } else {
             lab = __shfl(my_lab, g * LPR + p);
         }
+        const T* staged = reinterpret_cast<const T*>(stage);
+        const float xb = Elem<T>::to_f32(staged[blank]);
+        const float xl = Elem<T>::to_f32(staged[lab < 0 ? 0 : lab]);
         Lse lse;
-        float xb, xl;
-        gather_pass<T, LPR, K>(raw[p], g, pb, lab, lse, xb, xl);
+        float unused_b, unused_l;
+        gather_pass<T, LPR, K, false>(raw[p], g, pb, lab, lse, unused_b, unused_l);
         const bool here = lir == p;
         res_lse.m = here ? lse.m : res_lse.m;
         res_lse.l2s = here ? lse.l2s : res_lse.l2s;
