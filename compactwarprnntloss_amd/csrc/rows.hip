@@ -880,6 +880,37 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_flat(
     store_raw<NT>(gx + at, grad_pack<T, FUSED>(in, rc, pack, blank, V));
 }
 
+// Rows of 64/RP packs, RP = 2 or 4: a wave moves RP whole rows, one pack per lane, as one run of 64
+// consecutive packs.  The rows are wave-uniform, so their coefficients come through the scalar
+// unit and each lane selects its row's; per-lane loads of the row records (three more vector
+// loads per lane, most lanes asking for the same address) cost 5 % of the pass on 512-byte rows.
+template <typename T, bool FUSED, int RP, bool NT>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad_rows(
+    const T* __restrict__ x, i64 R, int V, int N, int blank, const int2* __restrict__ rowinfo,
+    const float2* __restrict__ grads, const float* __restrict__ lse, const GradOut grad_costs,
+    T* __restrict__ gx) {
+    constexpr int VEC = Elem<T>::VEC;
+    constexpr int LPR = 64 / RP;
+    const int lane = threadIdx.x & 63;
+    const i64 r0 = wave_first_row<true>(RP);
+    if (r0 >= R) return;
+    const int g = lane / LPR;
+    const bool ok = r0 + g < R;
+    const i64 at = (r0 * LPR + (ok ? lane : lane % LPR)) * VEC;  // rows beyond the tensor re-read the wave's first
+    v4i in = {0, 0, 0, 0};
+    if (FUSED) in = load_raw<NT>(x + at);
+    RowCoef rc = row_coef<FUSED>(r0, N, rowinfo, grads, lse, grad_costs);
+#pragma unroll
+    for (int j = 1; j < RP; ++j) {
+        const RowCoef cj = row_coef<FUSED>(r0 + j < R ? r0 + j : r0, N, rowinfo, grads, lse, grad_costs);
+        const bool mine = g == j;
+        rc.cg = mine ? cj.cg : rc.cg; rc.cb = mine ? cj.cb : rc.cb; rc.cl = mine ? cj.cl : rc.cl;
+        rc.nls = mine ? cj.nls : rc.nls; rc.lab = mine ? cj.lab : rc.lab;
+    }
+    const v4i o = grad_pack<T, FUSED>(in, rc, lane % LPR, blank, V);
+    if (ok) store_raw<NT>(gx + at, o);
+}
+
 // Other packed shapes: LPR lanes per row, K packs per lane, 64/LPR rows per wave.
 template <typename T, bool FUSED, int LPR, int K, bool NT>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void k_grad(
@@ -1081,6 +1112,17 @@ static int grad_typed(const Batch& b, const int* rowinfo, const float* grads, co
             CWR_LAUNCH((k_grad_flat<T, FUSED, kGradNT>), dim3((blocks_for_waves(b.R * ch) + 7u) & ~7u),
                                dim3(kWavesPerBlock * 64), 0, b.stream, x, b.R, b.V, b.N, b.blank, ch, ri, g2,
                                lse, grad_costs, gx);
+            return check_launch();
+        }
+        if ((NV == 32 || NV == 16) && (b.R + 1) / 2 < 0x7fffffffLL) {
+            const int rp = 64 / NV;
+            const unsigned blocks = (blocks_for_waves((b.R + rp - 1) / rp) + 7u) & ~7u;
+            if (rp == 2)
+                CWR_LAUNCH((k_grad_rows<T, FUSED, 2, kGradNT>), dim3(blocks), dim3(kWavesPerBlock * 64), 0, b.stream, x,
+                           b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);
+            else
+                CWR_LAUNCH((k_grad_rows<T, FUSED, 4, kGradNT>), dim3(blocks), dim3(kWavesPerBlock * 64), 0, b.stream, x,
+                           b.R, b.V, b.N, b.blank, ri, g2, lse, grad_costs, gx);
             return check_launch();
         }
         if (pick_shape(NV, &lpr, &k)) {
