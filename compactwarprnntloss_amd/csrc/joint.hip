@@ -477,9 +477,9 @@ __global__ __launch_bounds__(256, 2) void k_joint_dz(
 constexpr int kRK = 64;      // K-slice of the weight tile
 constexpr int kRPitch = 72;  // 144 bytes: 16 consecutive rows start in 16 different groups of four banks
 
-template <typename T> struct ResLds {
-    T w[2][kJN][kRPitch];
-    float bias[2][kJN];  // what the accumulators of a tile start from
+template <typename T, int NMV> struct ResLds {
+    T w[2][32 * NMV][kRPitch];
+    float bias[2][32 * NMV];  // what the accumulators of a tile start from
 };
 
 // this wave's data rows [row0, row0 + 32 ND), as MFMA operand fragments
@@ -499,10 +499,12 @@ __device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 
 }
 
 // tile(acc, v0) receives acc[mv][nd] = vocabulary entries [v0 + 32 mv, v0 + 32 mv + 32) x data rows
-// [32 nd, 32 nd + 32) of the wave's rows in hreg
-template <typename T, int ND, int KS, bool D2, typename TileFn>
+// [32 nd, 32 nd + 32) of the wave's rows in hreg; the vocabulary is walked in tiles of JN = 32 NMV
+template <typename T, int ND, int KS, int NMV, bool D2, typename TileFn>
 __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T* __restrict__ W,
-                                              const float* __restrict__ bias, int V, ResLds<T>& lds, TileFn&& tile) {
+                                              const float* __restrict__ bias, int V, ResLds<T, NMV>& lds,
+                                              TileFn&& tile) {
+    constexpr int JN = 32 * NMV;
     constexpr int H = KS * 16;
     constexpr int NK = H / kRK;  // K-slices per vocabulary tile
     static_assert(H % kRK == 0, "whole K-slices");
@@ -512,22 +514,22 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
     const int lane = tid & 63;
     const int hf = lane >> 5, l32 = lane & 31;
 
-    // ---- weight tile: thread t moves 16-byte piece (t % 8) of rows t / 8 + 32 p, p = 0..3 ----------
+    // ---- weight tile: thread t moves 16-byte piece (t % 8) of rows t / 8 + 32 p, p < NMV ----------
     const int st_row = tid >> 3, st_piece = tid & 7;
-    struct Pre { v4i w[4]; };
+    struct Pre { v4i w[NMV]; };
     Pre pre[D2 ? 2 : 1];
-    const int nvt = (V + kJN - 1) / kJN;
+    const int nvt = (V + JN - 1) / JN;
     auto fetch = [&](int vt, int kc, Pre& q) {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            int v = vt * kJN + st_row + 32 * p;
+        for (int p = 0; p < NMV; ++p) {
+            int v = vt * JN + st_row + 32 * p;
             if (v >= V) v = V - 1;  // entries beyond the vocabulary are masked in the accumulator
             q.w[p] = *reinterpret_cast<const v4i*>(W + (i64)v * H + kc * kRK + st_piece * 8);
         }
     };
     auto stage = [&](int buf, const Pre& q) {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + 32 * p][st_piece * 8]) = q.w[p];
+        for (int p = 0; p < NMV; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + 32 * p][st_piece * 8]) = q.w[p];
     };
 
     // slices are numbered it = vt * NK + kc; slice it is multiplied out of buffer it & 1 (NK is even
@@ -535,21 +537,21 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
     // the bias of a tile (-inf beyond the vocabulary, which no finite product changes and which drops
     // out of both the maximum and the sum) is fetched by the first 128 threads one tile ahead
     auto bias_of = [&](int vt) {
-        const int v = vt * kJN + tid;
+        const int v = vt * JN + tid;
         return v < V ? (bias ? bias[v] : 0.f) : -INFINITY;
     };
     float bias_next = 0.f;
-    if (tid < kJN) s_bias[0][tid] = bias_of(0);
+    if (tid < JN) s_bias[0][tid] = bias_of(0);
     fetch(0, 0, pre[0]);
     if (D2 && (NK > 1 || nvt > 1)) fetch(NK > 1 ? 0 : 1, NK > 1 ? 1 : 0, pre[1]);
     stage(0, pre[0]);
     __syncthreads();
 
-    f32x16 acc[4][ND];
+    f32x16 acc[NMV][ND];
     int par = 0;  // buffer of the current slice
     for (int vt = 0; vt < nvt; ++vt) {
 #pragma unroll
-        for (int mv = 0; mv < 4; ++mv)
+        for (int mv = 0; mv < NMV; ++mv)
 #pragma unroll
             for (int b4 = 0; b4 < 4; ++b4) {
                 const float4 bq = *reinterpret_cast<const float4*>(&s_bias[vt & 1][32 * mv + 8 * b4 + 4 * hf]);
@@ -559,10 +561,10 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
                     acc[mv][nd][4 * b4 + 2] = bq.z; acc[mv][nd][4 * b4 + 3] = bq.w;
                 }
             }
-        if (tid < kJN && vt + 1 < nvt) bias_next = bias_of(vt + 1);
+        if (tid < JN && vt + 1 < nvt) bias_next = bias_of(vt + 1);
 #pragma unroll
         for (int kc = 0; kc < NK; ++kc) {
-            if (kc == NK - 1 && tid < kJN && vt + 1 < nvt) s_bias[(vt + 1) & 1][tid] = bias_next;  // before its barrier
+            if (kc == NK - 1 && tid < JN && vt + 1 < nvt) s_bias[(vt + 1) & 1][tid] = bias_next;  // before its barrier
             // register set kc & 1 held this slice's loads (already staged); it now takes slice it + 2
             if (D2) {
                 const int k2 = kc + 2;
@@ -578,13 +580,13 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
             // register and pays the LDS latency in front of every matrix instruction).
 #pragma unroll
             for (int ks = 0; ks < kRK / 16; ++ks) {
-                v4i fa[4];
+                v4i fa[NMV];
 #pragma unroll
-                for (int mv = 0; mv < 4; ++mv)
+                for (int mv = 0; mv < NMV; ++mv)
                     fa[mv] = *reinterpret_cast<const v4i*>(&s_w[par][32 * mv + l32][16 * ks + 8 * hf]);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int mv = 0; mv < 4; ++mv)
+                for (int mv = 0; mv < NMV; ++mv)
 #pragma unroll
                     for (int nd = 0; nd < ND; ++nd)
                         acc[mv][nd] = Mfma<T>::mac(fa[mv], hreg[nd][kc * (kRK / 16) + ks], acc[mv][nd]);
@@ -598,17 +600,17 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
             __syncthreads();
             par ^= 1;
         }
-        tile(acc, vt * kJN);
+        tile(acc, vt * JN);
     }
 }
 
-template <typename T, int ND, int KS, int OCC, bool D2>
+template <typename T, int ND, int KS, int NMV, int OCC, bool D2>
 __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
     const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
     const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
     int blank, const FwdOut out, int* __restrict__ status) {
-    __shared__ __attribute__((aligned(16))) ResLds<T> lds;
+    __shared__ __attribute__((aligned(16))) ResLds<T, NMV> lds;
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
@@ -617,8 +619,8 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     load_resident_rows<T, ND, KS>(h, R, row0, hreg);
     FwdRows<ND> q;
     fwd_rows_init<ND>(q, row0 + l32, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
-    walk_resident<T, ND, KS, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[4][ND], int v0) {
-        fwd_fold_tile<4, ND>(acc, v0, blank, hf, q);
+    walk_resident<T, ND, KS, NMV, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[NMV][ND], int v0) {
+        fwd_fold_tile<NMV, ND>(acc, v0, blank, hf, q);
     });
     fwd_merge_halves<ND>(q);
 #pragma unroll
@@ -629,12 +631,12 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     }
 }
 
-template <typename T, int ND, int KS, int OCC, bool D2>
+template <typename T, int ND, int KS, int NMV, int OCC, bool D2>
 __global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
     const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V, int N, int blank,
     const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
     const GradOut go, T* __restrict__ dz) {
-    __shared__ __attribute__((aligned(16))) ResLds<T> lds;
+    __shared__ __attribute__((aligned(16))) ResLds<T, NMV> lds;
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
@@ -643,16 +645,18 @@ __global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
     load_resident_rows<T, ND, KS>(h, R, row0, hreg);
     DzRows<ND> q;
     dz_rows_init<ND>(q, row0 + l32, R, N, rowinfo, grads, lse, go);
-    walk_resident<T, ND, KS, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[4][ND], int v0) {
-        dz_store_tile<T, 4, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz);
+    walk_resident<T, ND, KS, NMV, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[NMV][ND], int v0) {
+        dz_store_tile<T, NMV, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz);
     });
 }
 
 // The joint sizes in use take the resident kernels; any other multiple of 32 the streaming ones.
 // Measured on R = 311449, V = 1024, H = 512 (bf16): one data block per wave at two waves per SIMD
-// 0.46 ms; two blocks per wave at one wave per SIMD 0.63 ms (registers spill); streaming kernel 0.63 ms.
-#define CWR_JOINT_SHAPES(X) X(2, 16, 1, true) X(2, 24, 1, true) X(1, 32, 2, false) X(1, 40, 1, true) \
-                            X(1, 48, 1, true) X(1, 64, 1, true)
+// 0.44 ms; two blocks per wave at one wave per SIMD with tiles of 128 entries 0.63 ms (registers
+// spill), with tiles of 64 entries 0.49 ms (half the LDS reads per matrix instruction, but a lone
+// wave per SIMD hides neither the LDS latency nor the tile's reduction); streaming kernel 0.63 ms.
+#define CWR_JOINT_SHAPES(X) X(2, 16, 4, 1, true) X(2, 24, 4, 1, true) X(1, 32, 4, 2, false) X(1, 40, 4, 1, true) \
+                            X(1, 48, 4, 1, true) X(1, 64, 4, 1, true)
 
 template <typename T>
 static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
@@ -660,11 +664,11 @@ static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOp
     const FwdOut out = {ws.lp, lse, reinterpret_cast<int2*>(rowinfo), reinterpret_cast<float2*>(grads), ws.seqmode};
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
-#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                           \
+#define CWR_JOINT_RES(ND, KS, NMV, OCC, D2)                                                                           \
     if (j.H == 16 * KS) {                                                                                        \
         const i64 blocks = (b.R + 128 * ND - 1) / (128 * ND);                                                    \
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                     \
-        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w,  \
+        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w,  \
                    j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,     \
                    b.N, b.blank, out, b.status);                                                                 \
         return check_launch();                                                                                   \
@@ -695,11 +699,11 @@ static int joint_dlogits_typed(const JointOperands& j, i64 R, int V, int N, int 
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
     T* dz = static_cast<T*>(dlogits);
-#define CWR_JOINT_RES(ND, KS, OCC, D2)                                                                          \
+#define CWR_JOINT_RES(ND, KS, NMV, OCC, D2)                                                                          \
     if (j.H == 16 * KS) {                                                                                       \
         const i64 blocks = (R + 128 * ND - 1) / (128 * ND);                                                     \
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                    \
-        CWR_LAUNCH((k_joint_dz_res<T, ND, KS, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, stream, h, w,    \
+        CWR_LAUNCH((k_joint_dz_res<T, ND, KS, NMV, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, stream, h, w,    \
                    j.bias, R, V, N, blank, ri, gr, lse, go, dz);                                                \
         return check_launch();                                                                                  \
     }
