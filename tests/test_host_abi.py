@@ -264,3 +264,29 @@ def test_cost_rule_matches_the_oracle_including_the_averaging_branch():
     got, rc = device_rule(-2e-7, -1e-7)
     assert want_mis and rc == 0 and abs(got - 1e-7) < 1e-12
     assert lib.cwr_cost_rule(0.0, 0.0, None) == -1
+
+
+def test_joint_entry_points_reject_invalid_calls_on_the_host():
+    """cwr_joint_forward / cwr_joint_backward judge their arguments before any HIP call: storage
+    type, joint dimension, blank, null and misaligned buffers.  Every call here fails that judgement (or
+    has nothing to do), so the fake addresses are never handed to a kernel."""
+    lib = _lib.load()
+    A = 1 << 20  # an aligned fake address
+
+    def bwd(dtype=_lib.BF16, R=100, H=64, V=40, N=2, blank=0, h=A, w=A, ri=A, g=A, lse=A, gc=A, stride=1, dz=A):
+        return lib.cwr_joint_backward(h, w, None, dtype, R, H, V, N, blank, ri, g, lse, gc, stride, 1.0, dz, None)
+
+    assert bwd(dtype=_lib.F32) == 2 and bwd(dtype=_lib.F64) == 2     # CWR_ERR_DTYPE: matrix cores take 16-bit inputs
+    assert bwd(H=48) == 4 and bwd(H=0) == 4 and bwd(R=-1) == 4 and bwd(V=0) == 4 and bwd(stride=2) == 4
+    assert bwd(blank=40) == 5 and bwd(blank=-1) == 5
+    assert bwd(R=0) == 0                                             # nothing to do, nothing touched
+    for name in ("h", "w", "ri", "g", "lse", "gc", "dz"):
+        assert bwd(**{name: None}) == 1, name
+    assert bwd(h=A + 8) == 6 and bwd(ri=A + 4) == 6 and bwd(dz=A + 4) == 6 and bwd(lse=A + 2) == 6
+    assert bwd(V=41, dz=A + 1) == 6      # (rows off the 8-byte grid only need element alignment)
+
+    def fwd(dtype=_lib.BF16, H=64, h=A, w=A):
+        return lib.cwr_joint_forward(h, w, None, dtype, 100, H, 40, A, A, A, 3, 6, 2, 0, 3, A, 1 << 20, A, A, A, A, A, A,
+                                     A, None)
+
+    assert fwd(dtype=_lib.F32) == 2 and fwd(H=40) == 4 and fwd(h=None) == 1 and fwd(w=A + 2) == 6
