@@ -36,7 +36,7 @@ struct Batch {
 // lattice_slot(); all values are base-2 logarithms.
 struct Workspace {
     i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
-    i64* slot_off;  // N+1  the same running sum without the -1 marks (monotone: searchable)
+    i64* slot_off;  // N+1  first chunk of each sequence in k_fill's work list (a running sum: searchable)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
     int* seqmode;   // N+1  per sequence: 0 = walked in the scaled linear domain; bit 0 = in the log domain
                     //      (gather's verdict), bits 1 / 2 = alpha / beta repeated in the log domain

@@ -57,21 +57,31 @@ __device__ __forceinline__ void buf_store_i32(__amdgpu_buffer_rsrc_t r, int voff
     __builtin_amdgcn_raw_buffer_store_b32(x, r, voff, soff, 0);
 }
 
+// k_fill works in chunks of kFillRows rows of one strip (its rows that hold cells: T + nl - 1 of
+// them); a sequence's chunks are numbered strip by strip.  Few rows per chunk: many short waves,
+// whose dependent loads (chunk -> sequence -> lattice values -> their scales) overlap across waves.
+constexpr int kFillRows = 4;
+__host__ __device__ __forceinline__ i64 strip_chunks(i64 T, i64 nl) { return (T + nl - 1 + kFillRows - 1) / kFillRows; }
+__host__ __device__ __forceinline__ i64 fill_chunks(i64 T, i64 Up) {
+    const i64 full = (Up - 1) >> 6;
+    return full * strip_chunks(T, 64) + strip_chunks(T, Up - (full << 6));
+}
+
 // ---------------------------------------------------------------------------------------------
 // offsets
 // ---------------------------------------------------------------------------------------------
-// One wave.  Four exclusive scans over the sequences: compact rows, labels, lattice slots and
-// boundary-stream entries.  A sequence the kernels cannot take (bad lengths, rows beyond R, more
+// One wave.  Five exclusive scans over the sequences: compact rows, labels, lattice slots,
+// boundary-stream entries and the chunks k_fill works in (fill_chunks).  A sequence the kernels cannot take (bad lengths, rows beyond R, more
 // labels than max_u) gets pad_off = -1 and cost = NaN, and is skipped everywhere.
 __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, const int* __restrict__ ly,
                                                 i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
                                                 i64* __restrict__ row_off, i64* __restrict__ lab_off,
-                                                i64* __restrict__ pad_off, i64* __restrict__ slot_off,
+                                                i64* __restrict__ pad_off, i64* __restrict__ fill_off,
                                                 i64* __restrict__ bnd_off, int* __restrict__ seqmode,
                                                 int* __restrict__ status, float* __restrict__ costs,
                                                 float* __restrict__ reduced) {
     const int lane = threadIdx.x;
-    i64 carry_r = 0, carry_l = 0, carry_p = 0, carry_b = 0;
+    i64 carry_r = 0, carry_l = 0, carry_p = 0, carry_b = 0, carry_f = 0;
     int flags = 0, usable = 0;
     for (i64 base = 0; base < N; base += 64) {
         const i64 i = base + lane;
@@ -104,6 +114,10 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
         }
         const i64 inc_p = wave_inclusive_scan(slots);
         const i64 inc_b = wave_inclusive_scan(bnd);
+        // whether the sequence is usable is known only after the scans it takes part in: a sequence
+        // dropped below keeps its chunks, and k_fill skips them by its pad_off
+        const i64 chunks = (ok && pad_off) ? fill_chunks(T, (i64)U + 1) : 0;
+        const i64 inc_f = wave_inclusive_scan(chunks);
         if (i < N) {
             row_off[i] = start;
             lab_off[i] = carry_l + inc_l - labs;
@@ -115,7 +129,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
                 }
                 pad_off[i] = ok ? ps : -1;
                 usable += ok ? 1 : 0;
-                slot_off[i] = ps;
+                fill_off[i] = carry_f + inc_f - chunks;
                 bnd_off[i] = bs;
                 seqmode[i] = 0;
             }
@@ -125,6 +139,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
         carry_l += __shfl(inc_l, 63);
         carry_p += __shfl(inc_p, 63);
         carry_b += __shfl(inc_b, 63);
+        carry_f += __shfl(inc_f, 63);
     }
     flags |= __shfl_xor(flags, 1);
     flags |= __shfl_xor(flags, 2);
@@ -138,7 +153,7 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
         lab_off[N] = carry_l;
         if (pad_off) {
             pad_off[N] = carry_p;
-            slot_off[N] = carry_p;
+            fill_off[N] = carry_f;
             bnd_off[N] = carry_b;
         }
         if (R >= 0 && carry_r != R) flags |= CWR_FLAG_ROWS_MISMATCH;
@@ -154,10 +169,10 @@ __global__ __launch_bounds__(64) void k_offsets(const int* __restrict__ lx, cons
 }
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode,
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* fill_off, i64* bnd_off, int* seqmode,
                    int* status, float* costs, float* reduced, hipStream_t stream) {
     CWR_LAUNCH(k_offsets, dim3(1), dim3(64), 0, stream, lx, ly, N, R, max_u, slot_cap, bnd_cap,
-                       row_off, lab_off, pad_off, slot_off, bnd_off, seqmode, status, costs, reduced);
+                       row_off, lab_off, pad_off, fill_off, bnd_off, seqmode, status, costs, reduced);
     return check_launch();
 }
 
@@ -783,6 +798,16 @@ struct LatticeView {
         const float mant = (float)__builtin_amdgcn_frexp_mant(x);
         return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
     }
+    // the same in two steps, so that a caller can have many loads in flight before it converts
+    __device__ __forceinline__ i64 scale_index(i64 base, int k, int nl, int l) const {
+        return (base >> 4) + (k / kPF) * nl + l;
+    }
+    __device__ __forceinline__ double convert(double x, int C) const {
+        if (!linear) return x;
+        const int ex = __builtin_amdgcn_frexp_exp(x);
+        const float mant = (float)__builtin_amdgcn_frexp_mant(x);
+        return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
+    }
     __device__ __forceinline__ double log2_at(int t, int u) const {
         const i64 slot = pad + lattice_slot(t, u, T, Up);
         const double x = v[slot];
@@ -824,129 +849,147 @@ __device__ __forceinline__ void finish_costs(bool wrote, int N, float* costs, fl
     }
 }
 
-// One thread per lattice SLOT, so that a wave reads alpha, beta and the cell records of 64
-// neighbouring slots (consecutive addresses; a thread per compact row would touch one cache line
-// per lane, the strip layout being diagonal to the row order).  The two successors of cell (t,u)
-// sit one strip row further: same column (t+1,u) and next column (t,u+1); only the last column of a
-// strip looks into the next strip.  The 8-byte results are scattered to the row order.
-__device__ __forceinline__ bool fill_slot(const int* __restrict__ lx, const int* __restrict__ ly,
-                                               const i64* __restrict__ row_off,
-                                               const i64* __restrict__ pad_off,
-                                               const i64* __restrict__ slot_off,
-                                               const int* __restrict__ seqmode, int N, i64 R,
-                                               const LpCell* __restrict__ lp,
-                                               const double* __restrict__ alpha, const double* __restrict__ beta,
-                                               const int* __restrict__ scale_a, const int* __restrict__ scale_b,
-                                               float2* __restrict__ grads, float* __restrict__ costs,
-                                               int* __restrict__ status) {
-    // returns whether this thread wrote its sequence's cost
-    const i64 slot = (i64)blockIdx.x * 256 + threadIdx.x;
-    // the sequence whose slots hold this one: the last n with slot_off[n] <= slot (skipped
-    // sequences have no slots)
-    int n = 0;
-    if (N <= 64) {
-        // lane i holds slot_off[i]; a wave's 64 slots start in one sequence and cross few
-        // boundaries, so one ballot and a short loop replace a chain of dependent loads
-        const int lane = threadIdx.x & 63;
-        const i64 total = slot_off[N];
-        const i64 mine = lane < N ? slot_off[lane] : 0x7fffffffffffffffLL;
-        const i64 s0 = slot - lane;
-        n = __popcll(__ballot(mine <= s0)) - 1;
-        unsigned long long inside = __ballot(mine > s0 && mine <= s0 + 63);
-        while (inside) {
-            const int i = __ffsll((long long)inside) - 1;
-            inside &= inside - 1;
-            const i64 b = ((i64)__builtin_amdgcn_readlane((int)(mine >> 32), i) << 32) |
-                          (unsigned)__builtin_amdgcn_readlane((int)mine, i);
-            if (slot >= b) n = i;
-        }
-        if (slot >= total) return false;
-    } else {
-        // the wave's first slot is placed by a search on the scalar unit; its lanes step on from
-        // there over the few boundaries inside the wave's 64 slots (wave-uniform loads)
-        const i64 s0 = (i64)blockIdx.x * 256 + (__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) << 6);
-        if (s0 >= slot_off[N]) return false;
-        int lo = 0, hi = N;
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (slot_off[mid] <= s0) lo = mid; else hi = mid;
-        }
-        n = lo;
-        for (int j = lo + 1; j < N; ++j) {
-            const i64 oj = slot_off[j];
-            if (oj > s0 + 63) break;
-            n += oj <= slot ? 1 : 0;
-        }
-        if (slot >= slot_off[N]) return false;
-    }
-    const i64 pad = pad_off[n];
-    if (pad < 0) return false;
-    const int T = lx[n], U = ly[n];
-    const int Up = U + 1;
-    const int S = (Up + 63) >> 6;
-    const i64 full = strip_rows(T, 64) * 64;
-    const i64 local = slot - pad;
-    i64 s64 = local / full;
-    const int s = (int)(s64 < S - 1 ? s64 : S - 1);
-    const int rem = (int)(local - (i64)s * full);
-    const int nl = s == S - 1 ? Up - (s << 6) : 64;
-    const int row = rem / nl;
-    const int l = rem - row * nl;
-    const int t = row - l - kRowShift, u = (s << 6) + l;
-    if (t < 0 || t >= T) return false;  // padding
-    const i64 r = row_off[n] + (i64)t * Up + u;
-    if (r >= R) return false;
-    const int mode = seqmode[n];
-    LatticeView A, Bv;
-    A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
-    Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
-    const i64 base = pad + (i64)s * full;
-    const int q = t + l;
-    const double a = A.at_slot(slot, base, q, nl, l);
-    const LpCell cell = lp[slot];
-    const double b00 = Bv.log2_at(0, 0);
-    // all values are base-2 logarithms
-    float gb = 0.f, gl = 0.f;
-    if (t < T - 1) {
-        gb = -fast_exp2((float)(a + Bv.at_slot(slot + nl, base, T + nl - 2 - (q + 1), nl, l) + (double)cell.l_blank - b00));
-    } else if (u == U) {
-        gb = -fast_exp2((float)(a + (double)cell.l_blank - b00));
-    }
-    if (u < U) {
-        const double bn = l + 1 < nl ? Bv.at_slot(slot + nl + 1, base, T + nl - 2 - (q + 1), nl, l + 1) : Bv.log2_at(t, u + 1);
-        gl = -fast_exp2((float)(a + bn + (double)cell.l_label - b00));
-    }
-    grads[r] = make_float2(gb, gl);
-    if (t == T - 1 && u == U) {
-        float cost;
-        if (cost_rule(a + (double)cell.l_blank, b00, &cost)) raise_flag(status, CWR_FLAG_FB_MISMATCH);
-        costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : cost;
-        return true;
-    }
-    return false;
-}
-
+// One wave per chunk: kFillRows consecutive rows of one strip of one sequence.  Which sequence,
+// strip and rows is the same for the whole wave, so the search through the chunk offsets and all
+// the index arithmetic run once per wave on the scalar unit; a lane keeps one column (64 / nl rows
+// share a pass when the strip is narrow), reads alpha, beta and the cell records of its slots at
+// consecutive addresses (the strip layout is diagonal to the row order) and scatters the 8-byte
+// results to the row order.  The two successors of cell (t,u) sit one strip row further: same column
+// (t+1,u) and next column (t,u+1); only the last column of a strip looks into the next strip.
+// The grid is fixed; waves stride over the chunks, whose number only the device knows.
 __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
                                                const i64* __restrict__ pad_off,
-                                               const i64* __restrict__ slot_off,
+                                               const i64* __restrict__ fill_off,
                                                const int* __restrict__ seqmode, int N, i64 R,
                                                const LpCell* __restrict__ lp,
                                                const double* __restrict__ alpha, const double* __restrict__ beta,
                                                const int* __restrict__ scale_a, const int* __restrict__ scale_b,
                                                float2* __restrict__ grads, float* costs, float* reduced,
                                                int* status) {
-    const bool wrote = fill_slot(lx, ly, row_off, pad_off, slot_off, seqmode, N, R, lp, alpha, beta, scale_a,
-                                 scale_b, grads, costs, status);
-    finish_costs(wrote, N, costs, reduced, status);
+    const int lane = threadIdx.x & 63;
+    const i64 total = fill_off[N];
+    const i64 nwaves = (i64)gridDim.x * 4;
+    const i64 first = (i64)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    // Up to 64 sequences: lane i fetches everything about sequence i up front; one ballot then places
+    // a chunk and cross-lane reads hand out its sequence's values (a search through memory followed
+    // by the per-sequence loads would be two more rounds of dependent loads in front of everything
+    // else the wave does, and this kernel is made of such rounds).
+    const bool tables = N <= 64;
+    i64 t_fill = 0x7fffffffffffffffLL, t_pad = -1, t_row = 0;
+    int t_T = 0, t_U = 0, t_mode = 0;
+    if (tables && lane < N) {
+        t_fill = fill_off[lane]; t_pad = pad_off[lane]; t_row = row_off[lane];
+        t_T = lx[lane]; t_U = ly[lane]; t_mode = seqmode[lane];
+    }
+    auto lane_i64 = [](i64 v, int i) {
+        return ((i64)__builtin_amdgcn_readlane((int)(v >> 32), i) << 32) | (unsigned)__builtin_amdgcn_readlane((int)v, i);
+    };
+    for (i64 c = first; c < total; c += nwaves) {
+        // the sequence of chunk c: fill_off[n] <= c < fill_off[n+1]
+        int n;
+        i64 pad, roff, f0;
+        int T, U, mode;
+        if (tables) {
+            n = __popcll(__ballot(t_fill <= c)) - 1;
+            pad = lane_i64(t_pad, n); roff = lane_i64(t_row, n); f0 = lane_i64(t_fill, n);
+            T = __builtin_amdgcn_readlane(t_T, n); U = __builtin_amdgcn_readlane(t_U, n);
+            mode = __builtin_amdgcn_readlane(t_mode, n);
+        } else {
+            int lo = 0, hi = N;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (fill_off[mid] <= c) lo = mid; else hi = mid;
+            }
+            n = lo;
+            pad = pad_off[n]; roff = row_off[n]; f0 = fill_off[n];
+            T = lx[n]; U = ly[n]; mode = seqmode[n];
+        }
+        bool wrote = false;
+        if (pad >= 0) {
+            const int Up = U + 1;
+            const int S = (Up + 63) >> 6;
+            const unsigned per_full = (unsigned)strip_chunks(T, 64);
+            const unsigned local = (unsigned)(c - f0);
+            unsigned s = local / per_full;
+            s = s < (unsigned)(S - 1) ? s : (unsigned)(S - 1);
+            const int q0 = (int)(local - s * per_full) * kFillRows;  // first row of the chunk (0 = the strip's first cell row)
+            const int nl = (int)s == S - 1 ? Up - ((int)s << 6) : 64;
+            const int Q = T + nl - 1;
+            const i64 full = strip_rows(T, 64) * 64;
+            const i64 base = pad + (i64)s * full;
+            // the strip after this one, for the cells of this strip's last column
+            const int nl2 = (int)s + 1 < S ? ((int)s + 2 == S ? Up - (((int)s + 1) << 6) : 64) : 1;
+            const i64 base2 = base + full;
+            LatticeView A, Bv;
+            A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
+            Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
+            const double b00 = Bv.log2_at(0, 0);  // all values are base-2 logarithms
+            const int rpp = 64 / nl;  // rows per pass
+            const int rr = lane / nl, l = lane - rr * nl;
+            const int u = ((int)s << 6) + l;
+            // every pass's loads go out before any of them is used: lanes without a cell read
+            // the strip's first cell row instead and drop the result
+            struct Raw { double a, bd, bn; LpCell cell; int ca, cbd, cbn; int t; bool ok; };
+            Raw raw[kFillRows];
+#pragma unroll
+            for (int pass = 0; pass < kFillRows; ++pass) {
+                Raw& w = raw[pass];
+                const int p0 = pass * rpp;
+                const int q = q0 + p0 + rr;
+                const int t = q - l;
+                w.ok = rr < rpp && p0 + rr < kFillRows && q < Q && t >= 0 && t < T;
+                const int qs = w.ok ? q : 0, ls = w.ok ? l : 0;
+                w.t = qs - ls;
+                const i64 slot = base + (i64)(qs + kRowShift) * nl + ls;
+                const int kb = max(T + nl - 2 - (qs + 1), 0);  // step of the beta walk that wrote strip row qs + 1
+                const bool inside = ls + 1 < nl || !w.ok || (int)s + 1 >= S;  // else: column 0 of the next strip, row t
+                const i64 slot_n = inside ? slot + nl + 1 : base2 + (i64)(w.t + kRowShift) * nl2;
+                w.a = alpha[slot];
+                w.cell = lp[slot];
+                w.bd = beta[slot + nl];
+                w.bn = beta[slot_n];
+                w.ca = w.cbd = w.cbn = 0;
+                if (A.linear) w.ca = scale_a[A.scale_index(base, qs, nl, ls)];
+                if (Bv.linear) {
+                    w.cbd = scale_b[Bv.scale_index(base, kb, nl, ls)];
+                    w.cbn = scale_b[inside ? Bv.scale_index(base, kb, nl, min(ls + 1, nl - 1))
+                                           : Bv.scale_index(base2, max(T + nl2 - 2 - w.t, 0), nl2, 0)];
+                }
+            }
+#pragma unroll
+            for (int pass = 0; pass < kFillRows; ++pass) {
+                const Raw& w = raw[pass];
+                const int t = w.t;
+                const i64 r = roff + (i64)t * Up + u;
+                if (!w.ok || r >= R) continue;
+                const double a = A.convert(w.a, w.ca);
+                float gb = 0.f, gl = 0.f;
+                if (t < T - 1) gb = -fast_exp2((float)(a + Bv.convert(w.bd, w.cbd) + (double)w.cell.l_blank - b00));
+                else if (u == U) gb = -fast_exp2((float)(a + (double)w.cell.l_blank - b00));
+                if (u < U) gl = -fast_exp2((float)(a + Bv.convert(w.bn, w.cbn) + (double)w.cell.l_label - b00));
+                grads[r] = make_float2(gb, gl);
+                if (t == T - 1 && u == U) {
+                    float cost;
+                    if (cost_rule(a + (double)w.cell.l_blank, b00, &cost)) raise_flag(status, CWR_FLAG_FB_MISMATCH);
+                    costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : cost;
+                    wrote = true;
+                }
+            }
+        }
+        finish_costs(wrote, N, costs, reduced, status);
+    }
 }
 
+// Waves k_fill is launched with: one GPU full of them (8 per SIMD), never more than the chunks a batch of R rows in N sequences can have (a chunk holds at least one
+// row of cells of the lattice, and every strip ends with one partly filled chunk).
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs,
                 float* reduced) {
     if (b.R == 0) return CWR_OK;
-    const i64 slots = ws.slot_cap;  // the device knows the exact count; threads beyond it leave at once
-    if ((slots + 255) / 256 > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
-    CWR_LAUNCH(k_fill, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
+    const i64 strips = (b.max_u + 64) / 64;
+    i64 waves = b.R / kFillRows + (i64)b.N * strips * 6 + 1;
+    if (waves > 8192) waves = 8192;
+    CWR_LAUNCH(k_fill, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
                        ws.pad_off, ws.slot_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
                        ws.scale_b, reinterpret_cast<float2*>(grads), costs, reduced, b.status);
     (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
