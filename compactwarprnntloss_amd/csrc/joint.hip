@@ -197,23 +197,78 @@ template <int ND> struct FwdRows {
     int lab[ND];
 };
 
+// The rows' labels, in two steps around the loads of the resident rows.  begin: for up to 64 sequences
+// lane i asks for everything about sequence i (one round of loads, the oldest in the queue);
+// finish: a ballot places the wave's first row, the lanes step over the few sequence boundaries
+// inside the wave's rows, cross-lane reads hand out the sequence's values, and the label itself is
+// the one dependent load (needed when the first tile is folded).  More sequences than lanes: the
+// rows are placed by a search through memory in begin.
+struct SeqTable {
+    i64 off, pad, lab;
+    int T, U;
+};
+
 template <int ND>
-__device__ __forceinline__ void fwd_rows_init(FwdRows<ND>& q, i64 rbase, i64 R, const int* __restrict__ lx,
-                                              const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride,
-                                              i64 y_len, const i64* __restrict__ row_off,
-                                              const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
-                                              int V, int* __restrict__ status) {
-    // (only the label is needed during the walk over the vocabulary; the row's place in its lattice
-    // is worked out again at the end rather than kept in registers all along)
+__device__ __forceinline__ SeqTable fwd_rows_begin(FwdRows<ND>& q, i64 rbase, i64 R, const int* __restrict__ lx,
+                                                   const int* __restrict__ ly, const int* __restrict__ y,
+                                                   i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
+                                                   const i64* __restrict__ lab_off, const i64* __restrict__ pad_off,
+                                                   int N, int V, int* __restrict__ status) {
+    SeqTable tb;
+    tb.off = 0x7fffffffffffffffLL; tb.pad = -1; tb.lab = 0; tb.T = 0; tb.U = 0;
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) { q.m[nd] = -INFINITY; q.s[nd] = 0.f; q.xl[nd] = 0.f; q.xb[nd] = 0.f; q.lab[nd] = kNoLabel; }
+    const int lane = threadIdx.x & 63;
+    if (N <= 64) {
+        if (lane < N) {
+            tb.off = row_off[lane]; tb.pad = pad_off[lane]; tb.lab = lab_off[lane];
+            tb.T = lx[lane]; tb.U = ly[lane];
+        }
+        return tb;
+    }
 #pragma unroll
     for (int nd = 0; nd < ND; ++nd) {
-        q.m[nd] = -INFINITY; q.s[nd] = 0.f; q.xl[nd] = 0.f; q.xb[nd] = 0.f;
         const i64 r = rbase + 32 * nd;
-        q.lab[nd] = kNoLabel;
         if (r < R) {
             const RowInfo ri = decode_row(r, R, row_off, lx, ly, N);
             if (ri.n >= 0 && pad_off[ri.n] >= 0) q.lab[nd] = fetch_label(ri, y, y_stride, y_len, lab_off, V, status);
         }
+    }
+    return tb;
+}
+
+__device__ __forceinline__ i64 lane_i64(i64 v, int src) {  // v of lane src (src may differ between lanes)
+    const int lo = __shfl((int)(v & 0xffffffffLL), src), hi = __shfl((int)(v >> 32), src);
+    return ((i64)hi << 32) | (i64)(unsigned)lo;
+}
+
+template <int ND>
+__device__ __forceinline__ void fwd_rows_finish(FwdRows<ND>& q, const SeqTable& tb, i64 row0, i64 rbase, i64 R,
+                                                const int* __restrict__ y, i64 y_stride, i64 y_len, int N, int V,
+                                                int* __restrict__ status) {
+    if (N > 64 || N <= 0) return;
+    const unsigned long long m = __ballot(tb.off <= row0);
+    const int n0 = m ? 63 - __clzll((long long)m) : 0;  // sequence of the wave's first row
+    const i64 r_last = row0 + 32 * ND - 1;
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        const i64 r = rbase + 32 * nd;
+        int n = n0;
+        for (int j = n0 + 1; j < N; ++j) {
+            const i64 oj = lane_i64(tb.off, j);
+            if (oj > r_last) break;
+            n += oj <= r ? 1 : 0;
+        }
+        const i64 off = lane_i64(tb.off, n), pad = lane_i64(tb.pad, n), labbase = lane_i64(tb.lab, n);
+        const int T = __shfl(tb.T, n), U = __shfl(tb.U, n);
+        const i64 rem = r - off;
+        const i64 cells = (i64)T * (i64)(U + 1);
+        if (r >= R || T <= 0 || U < 0 || rem < 0 || rem >= cells || off + cells > R || pad < 0) continue;
+        const int u = cells < 0x7fffffffLL ? (int)((unsigned)rem % (unsigned)(U + 1)) : (int)(rem % (U + 1));
+        if (u >= U) continue;
+        const i64 at = (y_stride >= 0 ? (i64)n * y_stride : labbase) + u;
+        const int lab = (at >= 0 && at < y_len && (y_stride < 0 || u < y_stride)) ? y[at] : -1;
+        if (lab < 0 || lab >= V) { raise_flag(status, CWR_FLAG_BAD_LABEL); q.lab[nd] = kBadLabel; } else q.lab[nd] = lab;
     }
 }
 
@@ -304,25 +359,43 @@ template <int ND> struct DzRows {
     int lab[ND];
 };
 
+// in two steps around the loads of the resident rows: the row records are requested first (begin);
+// the coefficients, which need one dependent load (the sequence's incoming gradient), are formed
+// once the rows' loads are out (finish)
+template <int ND> struct DzRaw {
+    int2 info[ND];
+    float2 g[ND];
+    float lse[ND];
+};
+
 template <int ND>
-__device__ __forceinline__ void dz_rows_init(DzRows<ND>& q, i64 rbase, i64 R, int N, const int2* __restrict__ rowinfo,
-                                             const float2* __restrict__ grads, const float* __restrict__ lse,
-                                             const GradOut go) {
+__device__ __forceinline__ void dz_rows_begin(DzRaw<ND>& w, i64 rbase, i64 R, const int2* __restrict__ rowinfo,
+                                              const float2* __restrict__ grads, const float* __restrict__ lse) {
 #pragma unroll
     for (int nd = 0; nd < ND; ++nd) {
         const i64 r = rbase + 32 * nd;
+        w.info[nd] = make_int2(-1, -1); w.g[nd] = make_float2(0.f, 0.f); w.lse[nd] = 0.f;
+        if (r >= R) continue;
+        w.info[nd] = rowinfo[r]; w.g[nd] = grads[r]; w.lse[nd] = lse[r];
+    }
+}
+
+template <int ND>
+__device__ __forceinline__ void dz_rows_finish(DzRows<ND>& q, const DzRaw<ND>& w, i64 rbase, i64 R, int N,
+                                               const GradOut go) {
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
         q.cg[nd] = 0.f; q.cb[nd] = 0.f; q.cl[nd] = 0.f; q.lab[nd] = -1;
         q.nls[nd] = -INFINITY;  // a row of no usable sequence: 2^-inf * 0 = 0 whatever its logits
-        if (r >= R) continue;
-        const int2 info = rowinfo[r];
-        if (info.y < 0 || info.y >= N) continue;
+        const int2 info = w.info[nd];
+        if (rbase + 32 * nd >= R || info.y < 0 || info.y >= N) continue;
         const float g = go.p[(i64)info.y * go.stride] * go.scale;
-        const float2 gr = grads[r];
+        const float2 gr = w.g[nd];
         q.lab[nd] = info.x;
         q.cb[nd] = gr.x * g;
         q.cl[nd] = info.x >= 0 ? gr.y * g : 0.f;
         q.cg[nd] = -(gr.x + (info.x >= 0 ? gr.y : 0.f)) * g;
-        q.nls[nd] = -lse[r] * kLog2e;
+        q.nls[nd] = -w.lse[nd] * kLog2e;
     }
 }
 
@@ -416,7 +489,8 @@ __global__ __launch_bounds__(256, 2) void k_joint_fwd(
     const i64 rbase = row0 + 128 * wd + l32;  // the rows this lane reduces: rbase + 32 nd, nd = 0..3
 
     FwdRows<4> q;
-    fwd_rows_init<4>(q, rbase, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
+    const SeqTable tb = fwd_rows_begin<4>(q, rbase, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
+    fwd_rows_finish<4>(q, tb, row0 + 128 * wd, rbase, R, y, y_stride, y_len, N, V, status);
     walk_streaming<T>(h, W, bias, R, H, V, row0, lds,
                       [&](const f32x16 (&acc)[2][4], int v_wave) { fwd_fold_tile<2, 4>(acc, v_wave, blank, hf, q); });
 
@@ -457,7 +531,9 @@ __global__ __launch_bounds__(256, 2) void k_joint_dz(
     const i64 row0 = (i64)blockIdx.x * kJM;
     const i64 rbase = row0 + 128 * wd + l32;
     DzRows<4> q;
-    dz_rows_init<4>(q, rbase, R, N, rowinfo, grads, lse, go);
+    DzRaw<4> raw;
+    dz_rows_begin<4>(raw, rbase, R, rowinfo, grads, lse);
+    dz_rows_finish<4>(q, raw, rbase, R, N, go);
     walk_streaming<T>(h, W, bias, R, H, V, row0, lds, [&](const f32x16 (&acc)[2][4], int v_wave) {
         dz_store_tile<T, 2, 4>(acc, v_wave, V, blank, hf, rbase, row0 + 128 * wd + 128, R, q, dz);
     });
@@ -476,6 +552,14 @@ __global__ __launch_bounds__(256, 2) void k_joint_dz(
 // indexed statically).
 constexpr int kRK = 64;      // K-slice of the weight tile
 constexpr int kRPitch = 72;  // 144 bytes: 16 consecutive rows start in 16 different groups of four banks
+
+// Workgroup barrier that waits for this wave's LDS traffic only, never for the global loads it has in
+// flight (a __syncthreads() drains those too: the weight loads issued ahead, and at the start of
+// a workgroup the loads of the resident rows).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0); vmcnt and expcnt untouched
+    __builtin_amdgcn_s_barrier();
+}
 
 template <typename T, int NMV> struct ResLds {
     T w[2][32 * NMV][kRPitch];
@@ -499,11 +583,16 @@ __device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 
 }
 
 // tile(acc, v0) receives acc[mv][nd] = vocabulary entries [v0 + 32 mv, v0 + 32 mv + 32) x data rows
-// [32 nd, 32 nd + 32) of the wave's rows in hreg; the vocabulary is walked in tiles of JN = 32 NMV
-template <typename T, int ND, int KS, int NMV, bool D2, typename TileFn>
-__device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T* __restrict__ W,
+// [row0 + 32 nd, row0 + 32 nd + 32) of this wave; the vocabulary is walked in tiles of JN = 32 NMV.
+// Order of the start-up, which every workgroup of a round runs at the same time as every other: the
+// first weight slice is requested, then the resident rows (from HBM), then after_issue() runs
+// (what the caller still has to do about its rows: loads issued here queue up BEHIND the rows',
+// whatever the caller asked for earlier is served before them), and the first tile starts as
+// soon as the first fragments are there.
+template <typename T, int ND, int KS, int NMV, bool D2, typename AfterIssue, typename TileFn>
+__device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i64 row0, const T* __restrict__ W,
                                               const float* __restrict__ bias, int V, ResLds<T, NMV>& lds,
-                                              TileFn&& tile) {
+                                              AfterIssue&& after_issue, TileFn&& tile) {
     constexpr int JN = 32 * NMV;
     constexpr int H = KS * 16;
     constexpr int NK = H / kRK;  // K-slices per vocabulary tile
@@ -542,14 +631,20 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
     };
     float bias_next = 0.f;
     if (tid < JN) s_bias[0][tid] = bias_of(0);
+    v4i hreg[ND][KS];
+    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
+    after_issue();
     fetch(0, 0, pre[0]);
     if (D2 && (NK > 1 || nvt > 1)) fetch(NK > 1 ? 0 : 1, NK > 1 ? 1 : 0, pre[1]);
     stage(0, pre[0]);
-    __syncthreads();
+    lds_barrier();
 
     f32x16 acc[NMV][ND];
     int par = 0;  // buffer of the current slice
-    for (int vt = 0; vt < nvt; ++vt) {
+    // one vocabulary tile.  The first is a copy of its own: it follows the loads of the resident rows
+    // in straight-line code, so its K-steps wait for the fragments they use, one after the other,
+    // instead of for all of them in front of the loop.
+    auto one_tile = [&](const int vt) {
 #pragma unroll
         for (int mv = 0; mv < NMV; ++mv)
 #pragma unroll
@@ -597,11 +692,13 @@ __device__ __forceinline__ void walk_resident(const v4i (&hreg)[ND][KS], const T
                 const int vt1 = vt + k1 / NK;
                 if (vt1 < nvt) stage(par ^ 1, pre[D2 ? (kc + 1 + (NK & 1) * vt) & 1 : 0]);
             }
-            __syncthreads();
+            lds_barrier();
             par ^= 1;
         }
         tile(acc, vt * JN);
-    }
+    };
+    one_tile(0);
+    for (int vt = 1; vt < nvt; ++vt) one_tile(vt);
 }
 
 template <typename T, int ND, int KS, int NMV, int OCC, bool D2>
@@ -615,13 +712,13 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
     const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);  // first data row of this wave
-    v4i hreg[ND][KS];
-    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
     FwdRows<ND> q;
-    fwd_rows_init<ND>(q, row0 + l32, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V, status);
-    walk_resident<T, ND, KS, NMV, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[NMV][ND], int v0) {
-        fwd_fold_tile<NMV, ND>(acc, v0, blank, hf, q);
-    });
+    const SeqTable tb = fwd_rows_begin<ND>(q, row0 + l32, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V,
+                                           status);
+    fwd_rows_finish<ND>(q, tb, row0, row0 + l32, R, y, y_stride, y_len, N, V, status);
+    walk_resident<T, ND, KS, NMV, D2>(
+        h, R, row0, W, bias, V, lds, [&]() {},
+        [&](const f32x16 (&acc)[NMV][ND], int v0) { fwd_fold_tile<NMV, ND>(acc, v0, blank, hf, q); });
     fwd_merge_halves<ND>(q);
 #pragma unroll
     for (int nd = 0; nd < ND; ++nd) {
@@ -641,13 +738,14 @@ __global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
     const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);
-    v4i hreg[ND][KS];
-    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
     DzRows<ND> q;
-    dz_rows_init<ND>(q, row0 + l32, R, N, rowinfo, grads, lse, go);
-    walk_resident<T, ND, KS, NMV, D2>(hreg, W, bias, V, lds, [&](const f32x16 (&acc)[NMV][ND], int v0) {
-        dz_store_tile<T, NMV, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz);
-    });
+    DzRaw<ND> raw;
+    dz_rows_begin<ND>(raw, row0 + l32, R, rowinfo, grads, lse);
+    walk_resident<T, ND, KS, NMV, D2>(
+        h, R, row0, W, bias, V, lds, [&]() { dz_rows_finish<ND>(q, raw, row0 + l32, R, N, go); },
+        [&](const f32x16 (&acc)[NMV][ND], int v0) {
+            dz_store_tile<T, NMV, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz);
+        });
 }
 
 // The joint sizes in use take the resident kernels; any other multiple of 32 the streaming ones.

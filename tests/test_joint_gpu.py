@@ -41,6 +41,8 @@ def reference(j, grad_out=None, want_dense=False):
     ([40, 33, 17], [12, 20, 5], 96, 300, True),           # a ragged last vocabulary tile, several workgroups
     ([50, 21], [30, 70], 256, 1024, False),               # eight tiles, two strips, no bias
     ([30, 14], [9, 3], 32, 40, True),                     # fewer entries than half a tile: a wave with no valid entry
+    ([61, 40], [33, 70], 512, 1000, True),                # the largest resident shape at two waves per SIMD
+    ([25, 31], [20, 9], 768, 257, False),                 # one wave per SIMD, a single odd entry in the last tile
 ])
 def test_joint_forward_matches_oracle(dtype, lx, ly, H, V, bias):
     import compactwarprnntloss_amd as pkg
