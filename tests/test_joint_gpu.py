@@ -149,3 +149,48 @@ def test_fused_joint_loss_gradients_match_oracle(dtype, reduction):
         lm = pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "mean")
     _, ref1 = reference(j)
     assert abs(float(lm) - ref1["costs"].mean()) <= LOSS_RTOL * ref1["costs"].mean()
+
+
+def test_joint_forward_with_more_sequences_than_lanes():
+    """More than 64 sequences: the kernels place their rows by a search through the offsets instead
+    of through per-lane sequence tables."""
+    import compactwarprnntloss_amd as pkg
+    rng = np.random.default_rng(11)
+    N = 75
+    lx = rng.integers(1, 6, N)
+    ly = rng.integers(0, 4, N)
+    j = make_joint(lx, ly, 64, 130, seed=5, dtype="bf16", scale=2.0)
+    z, ref = reference(j)
+    costs, st = pkg.joint_forward(j["h"].to(DEV), j["w"].to(DEV), j["b"].to(DEV), torch.from_numpy(j["lx"]).to(DEV),
+                                  torch.from_numpy(j["yp"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV), 0)
+    torch.cuda.synchronize()
+    assert int(st.status[0].item()) == 0
+    np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
+
+
+def test_joiner_module_loss_agrees_with_the_stored_logits_route():
+    """CompactJoiner.loss (output layer fused into the loss) against the same module's logits handed
+    to transducer_loss, in bf16: the stored route rounds the logits to bf16 before the loss, the fused
+    one does not, so the two agree to bf16 accuracy of the logits, not better."""
+    import compactwarprnntloss_amd as pkg
+    torch.manual_seed(3)
+    N, E, P, J, V = 3, 24, 16, 64, 96
+    lx = torch.tensor([9, 14, 6], dtype=torch.int32, device=DEV)
+    ly = torch.tensor([4, 7, 2], dtype=torch.int32, device=DEV)
+    enc = torch.randn(N, 14, E, device=DEV, dtype=torch.bfloat16)
+    pred = torch.randn(N, 8, P, device=DEV, dtype=torch.bfloat16)
+    y = torch.randint(1, V, (N, 7), dtype=torch.int32, device=DEV)
+    joiner = pkg.CompactJoiner(E, P, J, V).to(DEV).to(torch.bfloat16)
+    fused = joiner.loss(enc, pred, lx, y, ly, 0, "mean")
+    fused.backward()
+    got = [p.grad.float().clone() for p in joiner.parameters()]
+    joiner.zero_grad()
+    stored = pkg.transducer_loss(joiner(enc, pred, lx, ly), lx, y, ly, 0, "mean", fused_log_softmax=True)
+    stored.backward()
+    assert abs(float(fused.detach()) - float(stored.detach())) <= 2e-2 * abs(float(stored.detach()))
+    for a, p in zip(got, joiner.parameters()):
+        b = p.grad.float()
+        assert torch.isfinite(a).all()
+        cos = torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0)
+        assert float(cos) > 0.99, float(cos)
