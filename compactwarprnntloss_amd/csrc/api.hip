@@ -41,7 +41,7 @@ static int scratch_of_current_device(void** out) {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t pad_off, slot_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
+    size_t pad_off, fill_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
     i64 slot_cap, bnd_cap;
 };
 
@@ -61,7 +61,7 @@ static Layout layout_for(i64 N, i64 R, i64 max_u) {
     l.bnd_cap = r / 64 + (bnd_by_strips < bnd_by_rows ? bnd_by_strips : bnd_by_rows) + 1;
     size_t at = 0;
     l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
-    l.slot_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
+    l.fill_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.seqmode = at; at = align_up(at + (size_t)(n + 1) * sizeof(int));
     l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(LpCell));
@@ -83,7 +83,7 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
     if (bytes < l.total) return false;
     char* p = static_cast<char*>(base);
     ws->pad_off = reinterpret_cast<i64*>(p + l.pad_off);
-    ws->slot_off = reinterpret_cast<i64*>(p + l.slot_off);
+    ws->fill_off = reinterpret_cast<i64*>(p + l.fill_off);
     ws->bnd_off = reinterpret_cast<i64*>(p + l.bnd_off);
     ws->seqmode = reinterpret_cast<int*>(p + l.seqmode);
     ws->lp = reinterpret_cast<LpCell*>(p + l.lp);
@@ -247,7 +247,7 @@ static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const in
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
-                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.slot_off, ws.bnd_off, ws.seqmode, status, costs,
+                        reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.fill_off, ws.bnd_off, ws.seqmode, status, costs,
                         reduced, s);
     if (rc != CWR_OK) return rc;
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,

@@ -36,7 +36,7 @@ struct Batch {
 // lattice_slot(); all values are base-2 logarithms.
 struct Workspace {
     i64* pad_off;   // N+1  first lattice slot of each sequence (-1: sequence skipped)
-    i64* slot_off;  // N+1  first chunk of each sequence in k_fill's work list (a running sum: searchable)
+    i64* fill_off;  // N+1  first chunk of each sequence in k_fill's work list (a running sum: searchable)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
     int* seqmode;   // N+1  per sequence: 0 = walked in the scaled linear domain; bit 0 = in the log domain
                     //      (gather's verdict), bits 1 / 2 = alpha / beta repeated in the log domain
@@ -57,7 +57,7 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
 int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t* bytes);
 
 int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 slot_cap, i64 bnd_cap,
-                   i64* row_off, i64* lab_off, i64* pad_off, i64* slot_off, i64* bnd_off, int* seqmode, int* status,
+                   i64* row_off, i64* lab_off, i64* pad_off, i64* fill_off, i64* bnd_off, int* seqmode, int* status,
                    float* costs_or_null, float* reduced_or_null, hipStream_t stream);
 // grads (may be null): rows of skipped sequences get a zero record there
 int launch_gather(const Batch& b, const Workspace& ws, float* lse, int* rowinfo, float* grads);

@@ -990,7 +990,7 @@ int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* 
     i64 waves = b.R / kFillRows + (i64)b.N * strips * 6 + 1;
     if (waves > 8192) waves = 8192;
     CWR_LAUNCH(k_fill, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
-                       ws.pad_off, ws.slot_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
+                       ws.pad_off, ws.fill_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
                        ws.scale_b, reinterpret_cast<float2*>(grads), costs, reduced, b.status);
     (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
     return check_launch();
