@@ -15,14 +15,17 @@
 // The reference repository has no joiner; its callers hand stored logits to
 // cwarp_rnnt/__init__.py:32-73.
 //
-// Tiling (gfx950, wave64, v_mfma_f32_32x32x16 on 16-bit inputs with fp32 accumulation).  A
-// workgroup of four waves owns 256 compact rows and walks the vocabulary in tiles of 128; the two
-// operand tiles travel through LDS in K-slices of 32, the next slice's global loads in flight
-// while the current one is multiplied.  The product is formed TRANSPOSED, C^T = W_tile * h_tile^T:
-// in the accumulator layout of a 32x32 block a lane then holds 16 vocabulary entries of ONE data
-// row, so the running maximum and the sum of exponentials of a row are kept per lane with no
-// cross-lane traffic until the very end.  Waves split the tile 2 x 2: wave (wd, wv) multiplies the
-// data rows [128 wd, 128 wd + 128) with the vocabulary entries [64 wv, 64 wv + 64) of the tile.
+// gfx950, wave64, v_mfma_f32_32x32x16 on 16-bit inputs with fp32 accumulation.  The product is
+// formed TRANSPOSED, C^T = W_tile * h_tile^T: in the accumulator layout of a 32x32 block a lane then
+// holds 16 vocabulary entries of ONE data row, so the running maximum and the sum of exponentials of
+// a row (forward) and the row's gradient coefficients (backward) are per-lane values, with no
+// cross-lane traffic until the very end.  Two tilings share the per-tile work:
+//   resident   (the joint sizes in use) a wave keeps the operand fragments of its own 32 or 64 data
+//              rows in registers for the whole kernel and only the weight tile travels through LDS;
+//   streaming  (any H that is a multiple of 32) a workgroup of four waves owns 256 rows and walks the
+//              vocabulary in tiles of 128, both operand tiles through LDS in K-slices of 32; waves
+//              split the tile 2 x 2: wave (wd, wv) multiplies the data rows [128 wd, 128 wd + 128)
+//              with the vocabulary entries [64 wv, 64 wv + 64) of the tile.
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
@@ -33,6 +36,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+// streaming tiling
 constexpr int kJM = 256;     // data rows per workgroup
 constexpr int kJN = 128;     // vocabulary entries per tile
 constexpr int kJK = 32;      // K-slice

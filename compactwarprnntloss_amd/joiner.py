@@ -5,7 +5,9 @@ of encoder frames and predictor states, run the output layer over all of it and 
 to cwarp_rnnt/__init__.py:52-59.  `compact_join` forms the sum for the cells of each sequence's own
 lattice only, directly in the compact row order of test/test.py:44-46 (kernels in csrc/join.hip,
 entry points cwr_join / cwr_join_backward); the output layer is then a plain GEMM over (R, H) rows,
-which `CompactJoiner` leaves to torch (hipBLASLt)."""
+which `CompactJoiner.forward` leaves to torch (hipBLASLt).  `fused_joint_loss` / `CompactJoiner.loss`
+go one step further for fp16 / bf16: the output layer is multiplied on the matrix cores inside the
+loss (csrc/joint.hip, cwr_joint_forward / cwr_joint_backward) and the (R, V) logits are never stored."""
 from typing import Any, Optional
 
 import torch
