@@ -423,9 +423,9 @@ template <> struct Pack4<__half> {
 // of ONE row, 32 rows side by side: 8-byte stores 2 V bytes apart) into whole rows: written as the
 // lanes hold it, read back with 16 lanes per row, stored as 64 NMV contiguous bytes per row.  Without
 // it the stores cost a fifth of the kernel (0.60 -> 0.49 ms with the stores removed).
-template <typename T, int NMV> struct DzTranspose {
+template <typename T, int NMV, int WAVES = 4> struct DzTranspose {
     static constexpr int kPitch = 32 * NMV + 8;  // elements; rows stay 16-byte aligned
-    T rows[4][32 * kPitch];
+    T rows[WAVES][32 * kPitch];
 };
 
 // acc[mv][nd] as in fwd_fold_tile; rbase = the lane's data row of nd = 0.  A lane holds runs of four
@@ -576,8 +576,8 @@ __global__ __launch_bounds__(256, 2) void k_joint_dz(
 // only the weight tile travels through LDS, in K-slices of 64, and every wave multiplies its rows
 // with the whole tile of 128 vocabulary entries.  Needs H known at compile time (the fragments are
 // indexed statically).
-constexpr int kRK = 64;      // K-slice of the weight tile
-constexpr int kRPitch = 72;  // 144 bytes: 16 consecutive rows start in 16 different groups of four banks
+// (the weight tile's K-slice RK is a parameter; its LDS rows are RK + 8 elements apart: 16 bytes past a
+// multiple of 128, so that 8 consecutive rows start in 8 different groups of four banks)
 
 // Workgroup barrier that waits for this wave's LDS traffic only, never for the global loads it has in
 // flight (a __syncthreads() drains those too: the weight loads issued ahead, and at the start of
@@ -587,8 +587,8 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_s_barrier();
 }
 
-template <typename T, int NMV> struct ResLds {
-    T w[2][32 * NMV][kRPitch];
+template <typename T, int NMV, int RK> struct ResLds {
+    T w[2][32 * NMV][RK + 8];
     float bias[2][32 * NMV];  // what the accumulators of a tile start from
 };
 
@@ -615,36 +615,41 @@ __device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 
 // (what the caller still has to do about its rows: loads issued here queue up BEHIND the rows',
 // whatever the caller asked for earlier is served before them), and the first tile starts as
 // soon as the first fragments are there.
-template <typename T, int ND, int KS, int NMV, bool D2, typename AfterIssue, typename TileFn>
+template <typename T, int ND, int KS, int NMV, int WAVES, int RK, bool D2, typename AfterIssue, typename TileFn>
 __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i64 row0, const T* __restrict__ W,
-                                              const float* __restrict__ bias, int V, ResLds<T, NMV>& lds,
+                                              const float* __restrict__ bias, int V, ResLds<T, NMV, RK>& lds,
                                               AfterIssue&& after_issue, TileFn&& tile) {
     constexpr int JN = 32 * NMV;
     constexpr int H = KS * 16;
-    constexpr int NK = H / kRK;  // K-slices per vocabulary tile
-    static_assert(H % kRK == 0, "whole K-slices");
+    constexpr int NK = H / RK;  // K-slices per vocabulary tile
+    static_assert(H % RK == 0, "whole K-slices");
     auto& s_w = lds.w;
     auto& s_bias = lds.bias;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int hf = lane >> 5, l32 = lane & 31;
 
-    // ---- weight tile: thread t moves 16-byte piece (t % 8) of rows t / 8 + 32 p, p < NMV ----------
-    const int st_row = tid >> 3, st_piece = tid & 7;
-    struct Pre { v4i w[NMV]; };
+    // ---- weight tile: a row of the slice is PPR pieces of 16 bytes; thread t moves piece t % PPR of rows
+    // t / PPR + RPP p ----------
+    constexpr int PPR = RK / 8;
+    constexpr int RPP = 64 * WAVES / PPR;  // rows the workgroup moves per pass
+    constexpr int NP = JN / RPP;           // passes per K-slice
+    static_assert(JN % RPP == 0, "whole passes");
+    const int st_row = tid / PPR, st_piece = tid % PPR;
+    struct Pre { v4i w[NP]; };
     Pre pre[D2 ? 2 : 1];
     const int nvt = (V + JN - 1) / JN;
     auto fetch = [&](int vt, int kc, Pre& q) {
 #pragma unroll
-        for (int p = 0; p < NMV; ++p) {
-            int v = vt * JN + st_row + 32 * p;
+        for (int p = 0; p < NP; ++p) {
+            int v = vt * JN + st_row + RPP * p;
             if (v >= V) v = V - 1;  // entries beyond the vocabulary are masked in the accumulator
-            q.w[p] = *reinterpret_cast<const v4i*>(W + (i64)v * H + kc * kRK + st_piece * 8);
+            q.w[p] = *reinterpret_cast<const v4i*>(W + (i64)v * H + kc * RK + st_piece * 8);
         }
     };
     auto stage = [&](int buf, const Pre& q) {
 #pragma unroll
-        for (int p = 0; p < NMV; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + 32 * p][st_piece * 8]) = q.w[p];
+        for (int p = 0; p < NP; ++p) *reinterpret_cast<v4i*>(&s_w[buf][st_row + RPP * p][st_piece * 8]) = q.w[p];
     };
 
     // slices are numbered it = vt * NK + kc; slice it is multiplied out of buffer it & 1 (NK is even
@@ -700,7 +705,7 @@ __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i6
             // instructions follow as they arrive (left to itself the compiler reuses ONE fragment
             // register and pays the LDS latency in front of every matrix instruction).
 #pragma unroll
-            for (int ks = 0; ks < kRK / 16; ++ks) {
+            for (int ks = 0; ks < RK / 16; ++ks) {
                 v4i fa[NMV];
 #pragma unroll
                 for (int mv = 0; mv < NMV; ++mv)
@@ -710,7 +715,7 @@ __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i6
                 for (int mv = 0; mv < NMV; ++mv)
 #pragma unroll
                     for (int nd = 0; nd < ND; ++nd)
-                        acc[mv][nd] = Mfma<T>::mac(fa[mv], hreg[nd][kc * (kRK / 16) + ks], acc[mv][nd]);
+                        acc[mv][nd] = Mfma<T>::mac(fa[mv], hreg[nd][kc * (RK / 16) + ks], acc[mv][nd]);
                 __builtin_amdgcn_sched_barrier(0);
             }
             {
@@ -727,22 +732,22 @@ __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i6
     for (int vt = 1; vt < nvt; ++vt) one_tile(vt);
 }
 
-template <typename T, int ND, int KS, int NMV, int OCC, bool D2>
-__global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
+template <typename T, int ND, int KS, int NMV, int WAVES, int RK, int OCC, bool D2>
+__global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_fwd_res(
     const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
     const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
     const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
     int blank, const FwdOut out, int* __restrict__ status) {
-    __shared__ __attribute__((aligned(16))) ResLds<T, NMV> lds;
+    __shared__ __attribute__((aligned(16))) ResLds<T, NMV, RK> lds;
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
-    const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);  // first data row of this wave
+    const i64 row0 = (i64)blockIdx.x * (32 * ND * WAVES) + (i64)w * (32 * ND);  // first data row of this wave
     FwdRows<ND> q;
     const SeqTable tb = fwd_rows_begin<ND>(q, row0 + l32, R, lx, ly, y, y_stride, y_len, row_off, lab_off, pad_off, N, V,
                                            status);
     fwd_rows_finish<ND>(q, tb, row0, row0 + l32, R, y, y_stride, y_len, N, V, status);
-    walk_resident<T, ND, KS, NMV, D2>(
+    walk_resident<T, ND, KS, NMV, WAVES, RK, D2>(
         h, R, row0, W, bias, V, lds, [&]() {},
         [&](const f32x16 (&acc)[NMV][ND], int v0) { fwd_fold_tile<NMV, ND>(acc, v0, blank, hf, q); });
     fwd_merge_halves<ND>(q);
@@ -754,22 +759,22 @@ __global__ __launch_bounds__(256, OCC) void k_joint_fwd_res(
     }
 }
 
-template <typename T, int ND, int KS, int NMV, int OCC, bool D2>
-__global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
+template <typename T, int ND, int KS, int NMV, int WAVES, int RK, int OCC, bool D2>
+__global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_dz_res(
     const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V, int N, int blank,
     const int2* __restrict__ rowinfo, const float2* __restrict__ grads, const float* __restrict__ lse,
     const GradOut go, T* __restrict__ dz) {
-    __shared__ __attribute__((aligned(16))) ResLds<T, NMV> lds;
+    __shared__ __attribute__((aligned(16))) ResLds<T, NMV, RK> lds;
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int hf = lane >> 5, l32 = lane & 31;
-    const i64 row0 = (i64)blockIdx.x * (128 * ND) + (i64)w * (32 * ND);
-    __shared__ __attribute__((aligned(16))) DzTranspose<T, NMV> tr;
+    const i64 row0 = (i64)blockIdx.x * (32 * ND * WAVES) + (i64)w * (32 * ND);
+    __shared__ __attribute__((aligned(16))) DzTranspose<T, NMV, WAVES> tr;
     T* tbuf = tr.rows[w];
     DzRows<ND> q;
     DzRaw<ND> raw;
     dz_rows_begin<ND>(raw, row0 + l32, R, rowinfo, grads, lse);
-    walk_resident<T, ND, KS, NMV, D2>(
+    walk_resident<T, ND, KS, NMV, WAVES, RK, D2>(
         h, R, row0, W, bias, V, lds, [&]() { dz_rows_finish<ND>(q, raw, row0 + l32, R, N, go); },
         [&](const f32x16 (&acc)[NMV][ND], int v0) {
             dz_store_tile<T, NMV, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz, tbuf);
@@ -777,12 +782,23 @@ __global__ __launch_bounds__(256, OCC) void k_joint_dz_res(
 }
 
 // The joint sizes in use take the resident kernels; any other multiple of 32 the streaming ones.
-// Measured on R = 311449, V = 1024, H = 512 (bf16): one data block per wave at two waves per SIMD
-// 0.44 ms; two blocks per wave at one wave per SIMD with tiles of 128 entries 0.63 ms (registers
-// spill), with tiles of 64 entries 0.49 ms (half the LDS reads per matrix instruction, but a lone
-// wave per SIMD hides neither the LDS latency nor the tile's reduction); streaming kernel 0.63 ms.
-#define CWR_JOINT_SHAPES(X) X(2, 16, 4, 1, true) X(2, 24, 4, 1, true) X(1, 32, 4, 2, false) X(1, 40, 4, 1, true) \
-                            X(1, 48, 4, 1, true) X(1, 64, 4, 1, true)
+// X(ND, H / 16, NMV, WAVES, RK, workgroups per CU, two register sets of weight loads in flight).
+// Measured on R = 311449, V = 1024, bf16, forward call (same GPU for every pair):
+//   eight waves per workgroup, one workgroup per CU, against four waves, two workgroups (the same
+//   two waves per SIMD, but one weight tile staged per 256 rows instead of per 128: half the L2
+//   traffic, staging instructions and LDS writes per matrix instruction):
+//       H = 256: 0.279 against 0.347 ms (two row blocks per wave, one wave per SIMD);
+//       H = 384: 0.365 against 0.418;  H = 512: 0.46 against 0.49;  H = 640: 0.59 against 0.67 ms;
+//       beyond H = 640 the fragments of 32 rows leave no room for two waves per SIMD;
+//   K-slices of 128 or 256 instead of 64 (fewer barriers): 0.465 / 0.49 against 0.467 ms at H = 512;
+//   two row blocks per wave at one wave per SIMD, H = 512: tiles of 128 entries 0.63 ms (registers
+//   spill), tiles of 64 entries 0.49 ms (half the LDS reads per matrix instruction, but a lone wave
+//   per SIMD hides neither the LDS latency nor the tile's reduction); streaming kernel 0.63 ms.
+//   the backward kernel follows, except at H = 512 (0.61 against 0.57 ms: it keeps four waves).
+#define CWR_JOINT_SHAPES(X) X(1, 16, 4, 8, 64, 1, true) X(1, 24, 4, 8, 64, 1, true) X(1, 32, 4, 8, 64, 1, false) \
+                            X(1, 40, 4, 8, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 64, 4, 4, 64, 1, true)
+#define CWR_JOINT_DZ_SHAPES(X) X(1, 16, 4, 8, 64, 1, true) X(1, 24, 4, 8, 64, 1, true) X(1, 32, 4, 4, 64, 2, false) \
+                               X(1, 40, 4, 8, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 64, 4, 4, 64, 1, true)
 
 template <typename T>
 static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
@@ -790,11 +806,11 @@ static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOp
     const FwdOut out = {ws.lp, lse, reinterpret_cast<int2*>(rowinfo), reinterpret_cast<float2*>(grads), ws.seqmode};
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
-#define CWR_JOINT_RES(ND, KS, NMV, OCC, D2)                                                                           \
+#define CWR_JOINT_RES(ND, KS, NMV, WAVES, RK, OCC, D2)                                                                           \
     if (j.H == 16 * KS) {                                                                                        \
-        const i64 blocks = (b.R + 128 * ND - 1) / (128 * ND);                                                    \
+        const i64 blocks = (b.R + 32 * ND * WAVES - 1) / (32 * ND * WAVES);                                                  \
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                     \
-        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w,  \
+        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, WAVES, RK, OCC, D2>), dim3((unsigned)blocks), dim3(64 * WAVES), 0, b.stream, h, w,  \
                    j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,     \
                    b.N, b.blank, out, b.status);                                                                 \
         return check_launch();                                                                                   \
@@ -825,15 +841,15 @@ static int joint_dlogits_typed(const JointOperands& j, i64 R, int V, int N, int 
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
     T* dz = static_cast<T*>(dlogits);
-#define CWR_JOINT_RES(ND, KS, NMV, OCC, D2)                                                                          \
+#define CWR_JOINT_RES(ND, KS, NMV, WAVES, RK, OCC, D2)                                                                          \
     if (j.H == 16 * KS) {                                                                                       \
-        const i64 blocks = (R + 128 * ND - 1) / (128 * ND);                                                     \
+        const i64 blocks = (R + 32 * ND * WAVES - 1) / (32 * ND * WAVES);                                                  \
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                    \
-        CWR_LAUNCH((k_joint_dz_res<T, ND, KS, NMV, OCC, D2>), dim3((unsigned)blocks), dim3(256), 0, stream, h, w,    \
+        CWR_LAUNCH((k_joint_dz_res<T, ND, KS, NMV, WAVES, RK, OCC, D2>), dim3((unsigned)blocks), dim3(64 * WAVES), 0, stream, h, w,    \
                    j.bias, R, V, N, blank, ri, gr, lse, go, dz);                                                \
         return check_launch();                                                                                  \
     }
-    CWR_JOINT_SHAPES(CWR_JOINT_RES)
+    CWR_JOINT_DZ_SHAPES(CWR_JOINT_RES)
 #undef CWR_JOINT_RES
     const i64 blocks = (R + kJM - 1) / kJM;
     if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
