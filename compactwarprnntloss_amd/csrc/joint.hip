@@ -293,12 +293,16 @@ __device__ __forceinline__ void fwd_fold_tile(const f32x16 (&acc)[NMV][ND], int 
         const float mn = fmaxf(q.m[nd], mx);
         if (mn > -INFINITY) {
             const float ms = mn * kLog2e;
-            float sum = q.s[nd] * fast_exp2(fmaf(q.m[nd], kLog2e, -ms));  // m = -inf: s = 0 stays 0
+            float sum = 0.f;
 #pragma unroll
             for (int mv = 0; mv < NMV; ++mv)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sum += fast_exp2(fmaf(acc[mv][nd][r], kLog2e, -ms));
-            q.s[nd] = sum;
+            // every exponent above is off by what ms lost to rounding (up to half an ulp of
+            // mn log2 e, the same for the whole tile): the fma recovers it exactly, so that s stays
+            // the sum of exp(x - m) and a row whose cost is tiny keeps its absolute accuracy
+            const float kept = q.m[nd] == mn ? q.s[nd] : q.s[nd] * fast_exp2((q.m[nd] - mn) * kLog2e);  // -inf: 0
+            q.s[nd] = fmaf(sum, fmaf(-fmaf(mn, kLog2e, -ms), kLn2, 1.f), kept);
             q.m[nd] = mn;
         }
         // the label's logit, if it sits in this lane's half of this part of the tile

@@ -169,6 +169,30 @@ def test_joint_forward_with_more_sequences_than_lanes():
     np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
 
 
+def test_joint_forward_keeps_the_absolute_accuracy_of_small_costs():
+    """Logits of large magnitude over small vocabularies: most rows are one-hot, row maxima are ~30
+    and a cost can be a few thousandths of a nat.  The running log-sum-exp of the tiles must not
+    inherit the rounding of maximum * log2(e) (half an ulp of ~40 per tile, 1e-6 nat)."""
+    import compactwarprnntloss_amd as pkg
+    rng = np.random.default_rng(77)
+    for case in range(36):
+        N = 16
+        lx = rng.integers(1, 6, N)
+        ly = rng.integers(0, 3, N)
+        V = [5, 40, 300][case % 3]                      # one tile, one tile, three tiles
+        H = [96, 64, 256][(case // 3) % 3]              # the streaming kernel and two resident shapes
+        j = make_joint(lx, ly, H, V, seed=int(rng.integers(1 << 30)), dtype=["f16", "bf16"][case % 2],
+                       scale=8.0, bias=bool(case & 4))
+        z, ref = reference(j)
+        costs, st = pkg.joint_forward(j["h"].to(DEV), j["w"].to(DEV), None if j["b"] is None else j["b"].to(DEV),
+                                      torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["yp"]).to(DEV),
+                                      torch.from_numpy(j["ly"]).to(DEV), 0)
+        torch.cuda.synchronize()
+        assert int(st.status[0].item()) == 0
+        np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL, atol=3e-7,
+                                   err_msg=f"case {case}: V={V} H={H}")
+
+
 def test_joiner_module_loss_agrees_with_the_stored_logits_route():
     """CompactJoiner.loss (output layer fused into the loss) against the same module's logits handed
     to transducer_loss, in bf16: the stored route rounds the logits to bf16 before the loss, the fused
