@@ -433,10 +433,10 @@ template <typename T, int NMV, int WAVES = 4> struct DzTranspose {
 };
 
 // acc[mv][nd] as in fwd_fold_tile; rbase = the lane's data row of nd = 0.  A lane holds runs of four
-// consecutive vocabulary entries of one row.  FAST: the whole tile lies inside the tensor, rows
-// start on 8-byte boundaries (V a multiple of 4) and the blank column is not in this part of the
-// tile: every run leaves as one unguarded 8-byte store.  Otherwise element by element, guarded.
-template <typename T, int NMV, int ND, bool FAST>
+// consecutive vocabulary entries of one row.  FAST: the whole tile lies inside the tensor and rows
+// start on 8-byte boundaries (V a multiple of 4): every run leaves as one unguarded 8-byte store.
+// Otherwise element by element, guarded.  BLANK: the blank column lies in this part of the tile.
+template <typename T, int NMV, int ND, bool FAST, bool BLANK>
 __device__ __forceinline__ void dz_store_tile_as(const f32x16 (&acc)[NMV][ND], int v_first, int V, int blank, int hf,
                                                  i64 rbase, i64 R, const DzRows<ND>& q, T* __restrict__ dz, T* tbuf) {
     constexpr int kTP = DzTranspose<T, NMV>::kPitch;
@@ -460,15 +460,15 @@ __device__ __forceinline__ void dz_store_tile_as(const f32x16 (&acc)[NMV][ND], i
                     const float p = fast_exp2(fmaf(acc[mv][nd][4 * b4 + c], kLog2e, q.nls[nd]));
                     o[c] = fmaf(p, q.cg[nd], key == e0 + c ? q.cl[nd] : 0.f);
                 }
+                if (BLANK && bl >= e0 && bl < e0 + 8) {  // it lies in this run of one of the two halves
+                    const int cb_at = bl - e0 - 4 * hf;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) o[c] += c == cb_at ? q.cb[nd] : 0.f;
+                }
                 if (FAST) {
                     if (tbuf) *reinterpret_cast<uint2*>(tbuf + l32 * kTP + e0 + 4 * hf) = Pack4<T>::of(o);
                     else *reinterpret_cast<uint2*>(row + e0) = Pack4<T>::of(o);
                     continue;
-                }
-                if (bl >= e0 && bl < e0 + 8) {  // the blank column lies in this run of one of the two halves
-                    const int cb_at = bl - e0 - 4 * hf;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) o[c] += c == cb_at ? q.cb[nd] : 0.f;
                 }
                 if (r >= R) continue;
                 const int v = v_first + 4 * hf + e0;
@@ -494,10 +494,12 @@ template <typename T, int NMV, int ND>
 __device__ __forceinline__ void dz_store_tile(const f32x16 (&acc)[NMV][ND], int v_first, int V, int blank, int hf,
                                               i64 rbase, i64 wave_rows_end, i64 R, const DzRows<ND>& q,
                                               T* __restrict__ dz, T* tbuf) {
-    const bool fast = (V & 3) == 0 && v_first + 32 * NMV <= V && wave_rows_end <= R &&
-                      (blank < v_first || blank >= v_first + 32 * NMV);
-    if (fast) dz_store_tile_as<T, NMV, ND, true>(acc, v_first, V, blank, hf, rbase, R, q, dz, (V & 7) == 0 ? tbuf : nullptr);
-    else dz_store_tile_as<T, NMV, ND, false>(acc, v_first, V, blank, hf, rbase, R, q, dz, nullptr);
+    const bool fast = (V & 3) == 0 && v_first + 32 * NMV <= V && wave_rows_end <= R;
+    const bool has_blank = blank >= v_first && blank < v_first + 32 * NMV;
+    T* const tb = (V & 7) == 0 ? tbuf : nullptr;
+    if (fast && !has_blank) dz_store_tile_as<T, NMV, ND, true, false>(acc, v_first, V, blank, hf, rbase, R, q, dz, tb);
+    else if (fast) dz_store_tile_as<T, NMV, ND, true, true>(acc, v_first, V, blank, hf, rbase, R, q, dz, tb);
+    else dz_store_tile_as<T, NMV, ND, false, true>(acc, v_first, V, blank, hf, rbase, R, q, dz, nullptr);
 }
 
 // ---------------------------------------------------------------------------------------------
