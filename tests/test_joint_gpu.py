@@ -193,6 +193,61 @@ def test_joint_forward_keeps_the_absolute_accuracy_of_small_costs():
                                    err_msg=f"case {case}: V={V} H={H}")
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_joint_random_shapes_against_oracle(seed):
+    """Fifteen random cases per seed: batch sizes on both sides of 64 sequences, joint sizes with and
+    without a resident kernel, vocabularies on and off the tile and store grids, both 16-bit types,
+    any blank, with and without bias, three logit scales, several block sizes of the backward pass:
+    costs, per-row gradients and the dense logit gradient against the oracle."""
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd import _lib
+    from compactwarprnntloss_amd.loss import _DTYPES, _stream_ptr
+    lib = _lib.load()
+    rng = np.random.default_rng(31000 + seed)
+    for case in range(15):
+        N = int(rng.integers(65, 80)) if rng.random() < 0.15 else int(rng.integers(1, 6))
+        lx = rng.integers(1, 40 if N < 10 else 6, N)
+        ly = rng.integers(0, 80 if (N < 10 and rng.random() < 0.3) else 12, N)
+        H = int(rng.choice([32, 64, 96, 256, 384, 512, 640, 768, 1024]))
+        V = int(rng.choice([5, 40, 128, 130, 256, 300, 515, 1024]))
+        dtype = str(rng.choice(["bf16", "f16"]))
+        blank = int(rng.integers(0, V))
+        scale = float(rng.choice([1.0, 3.0, 6.0]))
+        j = make_joint(lx, ly, H, V, seed=1000 * seed + case, dtype=dtype, scale=scale, bias=bool(rng.integers(0, 2)))
+        go = rng.uniform(0.5, 1.5, N)
+        what = f"seed {seed} case {case}: N={N} H={H} V={V} {dtype} blank={blank} scale={scale} R={j['R']}"
+        z = orc.joint_logits(j["h"].double().numpy(), j["w"].double().numpy(),
+                             None if j["b"] is None else j["b"].numpy())
+        ref = orc.loss_and_grad(z, j["lx"], j["yp"], j["ly"], blank, "fused", grad_out=go, want_dense=True)
+        h, W = j["h"].to(DEV), j["w"].to(DEV)
+        b = None if j["b"] is None else j["b"].to(DEV)
+        costs, st = pkg.joint_forward(h, W, b, torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["yp"]).to(DEV),
+                                      torch.from_numpy(j["ly"]).to(DEV), blank)
+        torch.cuda.synchronize()
+        assert int(st.status[0].item()) == 0, what
+        # a cost of a few thousandths of a nat carries the fp32 rounding of sums next to 1: 1e-7 absolute
+        np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL, atol=3e-7, err_msg=what)
+        np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL, err_msg=what)
+        R = j["R"]
+        gc = torch.from_numpy(go).float().to(DEV)
+        dz = torch.full((R, V), float("nan"), dtype=TDT[dtype], device=DEV)
+        block = int(rng.choice([R, 173, 1000]))
+        for r0 in range(0, R, block):
+            rc = lib.cwr_joint_backward(h[r0:].data_ptr(), W.data_ptr(), b.data_ptr() if b is not None else None,
+                                        _DTYPES[TDT[dtype]], min(block, R - r0), H, V, N, blank,
+                                        st.rowinfo[r0:].data_ptr(), st.grads[r0:].data_ptr(), st.lse[r0:].data_ptr(),
+                                        gc.data_ptr(), 1, 1.0, dz[r0:].data_ptr(), _stream_ptr(torch.device(DEV)))
+            assert rc == 0, (what, _lib.strerror(rc))
+        torch.cuda.synchronize()
+        got = dz.double().cpu().numpy()
+        eps = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+        # entries that are the difference of two terms (softmax * gamma against G) carry the fp32 rounding of both
+        tol = eps * np.abs(ref["grad"]) + 2e-5 * np.abs(ref["grad"]).max(axis=1, keepdims=True) + 5e-6
+        assert np.all(np.isfinite(got)), what
+        bad = np.abs(got - ref["grad"]) > tol
+        assert not bad.any(), (what, np.argwhere(bad)[:5], got[bad][:5], ref["grad"][bad][:5])
+
+
 def test_joiner_module_loss_agrees_with_the_stored_logits_route():
     """CompactJoiner.loss (output layer fused into the loss) against the same module's logits handed
     to transducer_loss, in bf16: the stored route rounds the logits to bf16 before the loss, the fused
