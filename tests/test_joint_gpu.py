@@ -248,6 +248,62 @@ def test_joint_random_shapes_against_oracle(seed):
         assert not bad.any(), (what, np.argwhere(bad)[:5], got[bad][:5], ref["grad"][bad][:5])
 
 
+def test_joint_full_size_config2_against_oracle():
+    """The fused output layer at the benchmark's own size (config 2's lengths, N=32, R=311449,
+    V=1024; H=512, bf16), sequence by sequence so that the float64 logits stay small: every cost
+    and every entry of the per-row gradients from cwr_joint_forward, and the logit gradient of
+    cwr_joint_backward (one call over all rows) on a few hundred sampled rows per sequence."""
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd import _lib, workloads as wl
+    from compactwarprnntloss_amd.loss import _DTYPES, _stream_ptr
+    cfg = wl.make_config(2)
+    N, R, V, H = cfg["N"], cfg["R"], cfg["V"], 512
+    g = torch.Generator(device="cpu").manual_seed(77)
+    h = torch.randn((R, H), generator=g).to(torch.bfloat16)
+    W = (torch.randn((V, H), generator=g) * (2.0 / H ** 0.5)).to(torch.bfloat16)   # logits ~ N(0, 2), as the config's
+    b = torch.randn(V, generator=g)
+    hd, Wd, bd = h.to(DEV), W.to(DEV), b.to(DEV)
+    lx, ly = torch.from_numpy(cfg["lx"]).to(DEV), torch.from_numpy(cfg["ly"]).to(DEV)
+    ys = torch.from_numpy(cfg["y_padded"]).to(DEV)
+    costs, st = pkg.joint_forward(hd, Wd, bd, lx, ys, ly, 0, max_u=ys.size(1))
+    rng = np.random.default_rng(5)
+    go = rng.uniform(0.5, 1.5, N) / N
+    gc = torch.from_numpy(go).float().to(DEV)
+    dz = torch.empty((R, V), dtype=torch.bfloat16, device=DEV)
+    rc = _lib.load().cwr_joint_backward(hd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), _DTYPES[torch.bfloat16], R, H, V,
+                                        N, 0, st.rowinfo.data_ptr(), st.grads.data_ptr(), st.lse.data_ptr(),
+                                        gc.data_ptr(), 1, 1.0, dz.data_ptr(), _stream_ptr(torch.device(DEV)))
+    assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    assert int(st.status[0].item()) == 0
+    costs = costs.cpu().numpy().astype(np.float64)
+    G_dev = st.grads.cpu().numpy().astype(np.float64)
+    off = orc.row_offsets_i64(cfg["lx"], cfg["ly"])
+    W64, b64 = W.double().numpy(), b.numpy()
+    for n in range(N):
+        a, e = int(off[n]), int(off[n + 1])
+        U = int(cfg["ly"][n])
+        z = orc.joint_logits(h[a:e].double().numpy(), W64, b64)
+        ref = orc.loss_and_grad(z, cfg["lx"][n:n + 1], cfg["y_padded"][n:n + 1], cfg["ly"][n:n + 1], 0, "fused",
+                                want_dense=False)
+        assert abs(costs[n] - ref["costs"][0]) <= LOSS_RTOL * abs(ref["costs"][0]), (n, costs[n], ref["costs"][0])
+        np.testing.assert_allclose(G_dev[a:e], ref["G"], rtol=0, atol=GRAD_ATOL, err_msg=f"sequence {n}")
+        gamma = -(ref["G"][:, 0] + ref["G"][:, 1])
+        rows = np.unique(np.concatenate([np.arange(U + 1), np.arange(e - a - U - 1, e - a),
+                                         rng.integers(0, e - a, 200)]))
+        want = np.exp(z[rows] - ref["lse"][rows, None]) * gamma[rows, None]
+        want[:, 0] += ref["G"][rows, 0]
+        u_of = rows % (U + 1)
+        has = u_of < U
+        lab = cfg["y_padded"][n, np.minimum(u_of, max(U - 1, 0))]
+        want[np.nonzero(has)[0], lab[has]] += ref["G"][rows[has], 1]
+        want *= go[n]
+        got = dz[torch.from_numpy(a + rows).to(DEV)].double().cpu().numpy()
+        tol = 2.0 ** -8 * np.abs(want) + 2e-5 * np.abs(want).max(axis=1, keepdims=True) + 1e-7
+        bad = np.abs(got - want) > tol
+        assert not bad.any(), (n, np.argwhere(bad)[:5], got[bad][:5], want[bad][:5])
+
+
 def test_joiner_module_loss_agrees_with_the_stored_logits_route():
     """CompactJoiner.loss (output layer fused into the loss) against the same module's logits handed
     to transducer_loss, in bf16: the stored route rounds the logits to bf16 before the loss, the fused
