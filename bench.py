@@ -325,6 +325,11 @@ def main():
             "forward_TFLOPs": round(flops / (fwd_call * 1e-3) / 1e12, 1),
             "dlogits_kernel_ms": round(dz_ms, 4),
             "dlogits_TFLOPs": round(flops / (dz_ms * 1e-3) / 1e12, 1),
+            # the one matrix-core kernel launched alone here: logits formed on MFMA (2 R H V flops per
+            # launch), turned into their gradient in registers and stored
+            "roofline": {"bound": "mfma", "kernel": "k_joint_dz (cwr_joint_backward)",
+                         "achieved": round(flops / (dz_ms * 1e-3) / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(flops / (dz_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
             "fwd_bwd_ms": round(fused_ms, 4),
             "fwd_bwd_TFLOPs": round(3 * flops / (fused_ms * 1e-3) / 1e12, 1),
             "fwd_bwd_frac_of_peak": round(3 * flops / (fused_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
