@@ -248,6 +248,41 @@ def test_joint_random_shapes_against_oracle(seed):
         assert not bad.any(), (what, np.argwhere(bad)[:5], got[bad][:5], ref["grad"][bad][:5])
 
 
+@pytest.mark.parametrize("H", [64, 256])
+def test_joint_bias_of_minus_inf_masks_a_vocabulary_entry(H):
+    """An entry switched off through its bias (-inf, no label uses it) drops out of every row's
+    log-sum-exp and gets a zero gradient; everything else matches the oracle on logits that hold
+    -inf in that column.  Both the streaming (H=64) and a resident (H=256) kernel."""
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd import _lib
+    from compactwarprnntloss_amd.loss import _DTYPES, _stream_ptr
+    V, off = 40, 15
+    j = make_joint([12, 7, 20], [4, 3, 9], H, V, seed=21, dtype="bf16", scale=2.0)
+    j["yp"][j["yp"] == off] = off - 1
+    j["b"][off] = -float("inf")
+    N, R = j["N"], j["R"]
+    with np.errstate(all="ignore"):
+        z = orc.joint_logits(j["h"].double().numpy(), j["w"].double().numpy(), j["b"].numpy())
+        ref = orc.loss_and_grad(z, j["lx"], j["yp"], j["ly"], 0, "fused", want_dense=True)
+    h, W, b = j["h"].to(DEV), j["w"].to(DEV), j["b"].to(DEV)
+    costs, st = pkg.joint_forward(h, W, b, torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["yp"]).to(DEV),
+                                  torch.from_numpy(j["ly"]).to(DEV), 0)
+    gc = torch.ones(N, device=DEV)
+    dz = torch.full((R, V), float("nan"), dtype=torch.bfloat16, device=DEV)
+    rc = _lib.load().cwr_joint_backward(h.data_ptr(), W.data_ptr(), b.data_ptr(), _DTYPES[torch.bfloat16], R, H, V, N,
+                                        0, st.rowinfo.data_ptr(), st.grads.data_ptr(), st.lse.data_ptr(),
+                                        gc.data_ptr(), 1, 1.0, dz.data_ptr(), _stream_ptr(torch.device(DEV)))
+    assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    assert int(st.status[0].item()) == 0
+    np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL)
+    got = dz.double().cpu().numpy()
+    assert np.all(np.isfinite(got)) and np.all(got[:, off] == 0)
+    tol = 2.0 ** -8 * np.abs(ref["grad"]) + 2e-5 * np.abs(ref["grad"]).max(axis=1, keepdims=True) + 1e-7
+    assert np.all(np.abs(got - ref["grad"]) <= tol)
+
+
 def test_joint_full_size_config2_against_oracle():
     """The fused output layer at the benchmark's own size (config 2's lengths, N=32, R=311449,
     V=1024; H=512, bf16), sequence by sequence so that the float64 logits stay small: every cost
