@@ -215,7 +215,9 @@ __global__ __launch_bounds__(256) void k_join_bwd_f(const T* __restrict__ dh, co
         if (r0 + cnt > R) cnt = R - r0;
         const T* pd = dh + r0 * H + col;
         const T* ph = h + r0 * H + col;
-#pragma unroll 4
+        // loads in flight per lane: twice as many rows at a time where there is no h to read beside dh
+        constexpr int kAhead = ACT == kActNone ? 8 : 4;
+#pragma unroll kAhead
         for (i64 u = 0; u < cnt; ++u) {
             const PackT<T, VEC> d = ld_stream<T, VEC>(pd + u * H);
             PackT<T, VEC> o;
@@ -255,7 +257,8 @@ __global__ __launch_bounds__(256) void k_join_bwd_g(const T* __restrict__ dh, co
         const T* pd = dh + r0 * H + col;
         const T* ph = h + r0 * H + col;
         const i64 stride = step * H;
-#pragma unroll 8
+        constexpr int kAhead = ACT == kActNone ? 16 : 8;
+#pragma unroll kAhead
         for (i64 t = 0; t < cnt; ++t) {
             const PackT<T, VEC> d = ld<T, VEC>(pd + t * stride);
             PackT<T, VEC> o;
