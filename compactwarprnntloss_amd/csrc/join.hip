@@ -92,10 +92,10 @@ __device__ __forceinline__ void st_stream(T* p, const PackT<T, VEC>& v) {
     }
 }
 
-// A wave takes kJoinRows consecutive compact rows; the first row's (n, t, u) is decoded on the
+// A wave takes JoinRows<T>::n consecutive compact rows; the first row's (n, t, u) is decoded on the
 // scalar unit and the following ones are stepped from it.  Only valid cells are visited, whatever
 // the padding of f and g.
-constexpr int kJoinRows = 4;
+template <typename T> struct JoinRows { static constexpr int n = sizeof(T) == 2 ? 8 : 4; };  // 16-bit rows are half as long
 
 template <typename T, int VEC, int ACT, bool FLAT>
 __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* __restrict__ g,
@@ -105,6 +105,7 @@ __global__ __launch_bounds__(256) void k_join(const T* __restrict__ f, const T* 
     typedef typename Arith<T>::type A;
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    constexpr int kJoinRows = JoinRows<T>::n;
     const i64 r0 = ((i64)blockIdx.x * 4 + w) * kJoinRows;
     if (r0 >= R) return;
     const int NV = H / VEC;
@@ -288,6 +289,7 @@ template <typename T, int VEC, int ACT>
 static int join_launch(const JoinArgs& j, bool backward) {
     if (!backward) {
         if (j.R == 0 || j.T_pad == 0 || j.Up_pad == 0) return CWR_OK;
+        constexpr int kJoinRows = JoinRows<T>::n;
         const i64 blocks = (j.R + 4 * kJoinRows - 1) / (4 * kJoinRows);
         if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
         if ((j.H / VEC) % 64 == 0)
