@@ -41,30 +41,33 @@ static int scratch_of_current_device(void** out) {
 static size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t pad_off, fill_off, bnd_off, seqmode, lp, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
+    size_t pad_off, fill_off, bnd_off, seqmode, lp, lpl, alpha, beta, scale_a, scale_b, bnd_a, bnd_b, aux, total;
     i64 slot_cap, bnd_cap;
 };
 
 // Upper bounds, from what the host knows (N, R, max_u), of the lattice slots and boundary-stream
-// entries a batch can need: every strip adds at most (63 + 2*kRowShift) * 64 padding slots to the
-// R real cells, and a sequence has at most ceil((max_u+1)/64) strips.
+// entries a batch can need: every strip adds at most (63 + 2*kRowShift) * 128 padding slots to the
+// R real cells (one padding row per lane but the first, and the rows in front and behind), a
+// sequence one slot to keep its size even, and a sequence has at most ceil((max_u+1)/128) strips.
 static Layout layout_for(i64 N, i64 R, i64 max_u) {
     Layout l;
     const i64 n = N > 0 ? N : 0, r = R > 0 ? R : 0, mu = max_u > 0 ? max_u : 0;
-    const i64 strips = (mu + 64) / 64;
-    i64 by_strips = r + n * strips * (63 + 2 * kRowShift) * 64;
-    i64 by_rows = r * (64 + 2 * kRowShift);  // each cell is also at most one full row of padding away
+    const i64 strips = strip_count(mu + 1);
+    i64 by_strips = r + n * (strips * (63 + 2 * kRowShift) * kStripCols + 1);
+    // each cell is also at most 63 + 2*kRowShift slots of padding away (a strip of one frame)
+    i64 by_rows = r * (64 + 2 * kRowShift) + n;
     l.slot_cap = by_strips < by_rows ? by_strips : by_rows;
     if (l.slot_cap < 0) l.slot_cap = 0;
-    // boundary streams: (S-1)*(T+kBndPad) per sequence, with (S-1)*64 <= U < rows of the sequence
+    // boundary streams: (S-1)*(T+kBndPad) per sequence, with (S-1)*128 <= U < rows of the sequence
     const i64 bnd_by_strips = n * (strips - 1) * kBndPad, bnd_by_rows = r * (kBndPad / 64);
-    l.bnd_cap = r / 64 + (bnd_by_strips < bnd_by_rows ? bnd_by_strips : bnd_by_rows) + 1;
+    l.bnd_cap = r / kStripCols + (bnd_by_strips < bnd_by_rows ? bnd_by_strips : bnd_by_rows) + 1;
     size_t at = 0;
     l.pad_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.fill_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.bnd_off = at; at = align_up(at + (size_t)(n + 1) * sizeof(i64));
     l.seqmode = at; at = align_up(at + (size_t)(n + 1) * sizeof(int));
-    l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(LpCell));
+    l.lp = at; at = align_up(at + (size_t)l.slot_cap * sizeof(float2));
+    l.lpl = at; at = align_up(at + (size_t)l.slot_cap * sizeof(float2));
     l.alpha = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
     l.beta = at; at = align_up(at + (size_t)l.slot_cap * sizeof(double));
     l.scale_a = at; at = align_up(at + ((size_t)l.slot_cap / 16 + 1) * sizeof(int));
@@ -86,7 +89,8 @@ bool carve_workspace(void* base, size_t bytes, i64 N, i64 R, i64 max_u, Workspac
     ws->fill_off = reinterpret_cast<i64*>(p + l.fill_off);
     ws->bnd_off = reinterpret_cast<i64*>(p + l.bnd_off);
     ws->seqmode = reinterpret_cast<int*>(p + l.seqmode);
-    ws->lp = reinterpret_cast<LpCell*>(p + l.lp);
+    ws->lp.p = reinterpret_cast<float2*>(p + l.lp);
+    ws->lp.l = reinterpret_cast<float2*>(p + l.lpl);
     ws->scale_a = reinterpret_cast<int*>(p + l.scale_a);
     ws->scale_b = reinterpret_cast<int*>(p + l.scale_b);
     ws->alpha = reinterpret_cast<double*>(p + l.alpha);
@@ -104,13 +108,14 @@ int workspace_section(i64 N, i64 R, i64 max_u, int which, size_t* offset, size_t
     if (N < 0 || R < 0 || max_u < 0) return CWR_ERR_SHAPE;
     Layout l = layout_for(N, R, max_u);
     switch (which) {
-        case 0: *offset = l.lp; *bytes = (size_t)l.slot_cap * sizeof(LpCell); return CWR_OK;
+        case 0: *offset = l.lp; *bytes = (size_t)l.slot_cap * sizeof(float2); return CWR_OK;
         case 1: *offset = l.alpha; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
         case 2: *offset = l.beta; *bytes = (size_t)l.slot_cap * sizeof(double); return CWR_OK;
         case 3: *offset = l.pad_off; *bytes = (size_t)(N + 1) * sizeof(i64); return CWR_OK;
         case 4: *offset = l.seqmode; *bytes = (size_t)(N + 1) * sizeof(int); return CWR_OK;
         case 5: *offset = l.scale_a; *bytes = ((size_t)l.slot_cap / 16 + 1) * sizeof(int); return CWR_OK;
         case 6: *offset = l.scale_b; *bytes = ((size_t)l.slot_cap / 16 + 1) * sizeof(int); return CWR_OK;
+        case 7: *offset = l.lpl; *bytes = (size_t)l.slot_cap * sizeof(float2); return CWR_OK;
     }
     return CWR_ERR_SHAPE;
 }

@@ -18,12 +18,13 @@ constexpr float kLn2 = 0.6931471805599453f;
 constexpr double kNeg = -1.0e30;
 constexpr float kLpFloor = -1.0e30f;  // gathered log-probs are clamped to this (keeps -inf logits finite)
 // The scaled linear-domain walk renormalises every kPF = 16 steps to a maximum of 2^kLinTarget
-// per column.  Inside a block a value can shrink by 2^(16*kLinMin) and grow by
-// 2^(16*(kLinMax+1)), which stays inside the fp64 range: 800 - 16*100 = -800 > -1022 and
-// 800 + 16*9 = 944 < 1023.
+// per lane.  A step multiplies a value by at most two factors (a lane walks two columns), each
+// within [2^kLinMin, 2^kLinMax], and adds at most doubles it: inside a block the largest value
+// stays below 2^(kLinTarget + 2*16*(kLinMax+1)) = 2^964, and the walk's own range check (every
+// second step) catches values that shrink towards the bottom of the fp64 range.
 constexpr float kLinMin = -100.0f;  // base-2 log-probs below this ...
-constexpr float kLinMax = 8.0f;     // ... or above this send the sequence to the log-domain walk
-constexpr int kLinTarget = 800;
+constexpr float kLinMax = 1.0f;     // ... or above this send the sequence to the log-domain walk
+constexpr int kLinTarget = 900;
 
 // ---------------------------------------------------------------------------------------------
 // wave64 cross-lane moves.  gfx9-family DPP controls.
@@ -165,37 +166,61 @@ template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PackT { T e[VEC];
 // layouts
 // ---------------------------------------------------------------------------------------------
 // Lattice storage (log-probs, alpha, beta).  A sequence's T x (U+1) lattice is cut into strips
-// of 64 label positions; strip s holds nl = min(64, U+1-64s) columns.  Inside a strip, cell
-// (t, u = 64s+l) is stored at row t+l+kRowShift, column l, of a dense (T+nl-1+2*kRowShift) x nl
-// array: a wave that walks the strip along its anti-diagonals touches one contiguous row per
-// step, at a constant pitch.  The rows above and below, and the two triangles of slots that hold
-// no cell, are padding.
+// of kStripCols = 128 label positions; strip s holds nl = min(128, U+1-128s) columns, two per lane
+// of the wave that walks it (lane j: columns 2j and 2j+1 of the strip).  Inside a strip, cell
+// (t, u = 128s+c) is stored at row t + c/2 + kRowShift, column c, of a dense
+// (T + ceil(nl/2) - 1 + 2*kRowShift) x nl array: a wave that walks the strip with lane j one frame
+// behind lane j-1 touches one contiguous row per step, at a constant pitch.  The rows above and
+// below, and the two triangles of slots that hold no cell, are padding.
 constexpr int kPF = 16;               // prefetch depth of the lattice walk, in rows
 constexpr int kRowShift = 2 * kPF;    // padding rows in front of (and behind) a strip
 constexpr int kBndPad = 192;          // entries a boundary stream holds beyond T
+constexpr int kStripCols = 128;       // label positions per strip
+constexpr int kStripShift = 7;        // log2(kStripCols)
 
-__host__ __device__ __forceinline__ i64 strip_rows(i64 T, i64 nl) { return T + nl - 1 + 2 * kRowShift; }
+__host__ __device__ __forceinline__ i64 strip_lanes(i64 nl) { return (nl + 1) >> 1; }
+__host__ __device__ __forceinline__ i64 strip_rows(i64 T, i64 nl) { return T + strip_lanes(nl) - 1 + 2 * kRowShift; }
+__host__ __device__ __forceinline__ i64 strip_count(i64 Up) { return (Up + kStripCols - 1) >> kStripShift; }
 __host__ __device__ __forceinline__ i64 lattice_slots(i64 T, i64 Up) {
-    i64 full = (Up - 1) >> 6;  // strips before the last one are 64 wide
-    i64 nl = Up - (full << 6);
-    return full * strip_rows(T, 64) * 64 + strip_rows(T, nl) * nl;
+    i64 full = (Up - 1) >> kStripShift;  // strips before the last one are full
+    i64 nl = Up - (full << kStripShift);
+    // an even number of slots: every strip then starts on a 16-byte boundary of the fp64 arrays
+    return (full * strip_rows(T, kStripCols) * kStripCols + strip_rows(T, nl) * nl + 1) & ~(i64)1;
 }
 __host__ __device__ __forceinline__ i64 lattice_slot(i64 t, i64 u, i64 T, i64 Up) {
-    i64 s = u >> 6, l = u & 63;
-    i64 nl = Up - (s << 6) < 64 ? Up - (s << 6) : 64;
-    return s * strip_rows(T, 64) * 64 + (t + l + kRowShift) * nl + l;
+    i64 s = u >> kStripShift, c = u & (kStripCols - 1);
+    i64 nl = Up - (s << kStripShift) < kStripCols ? Up - (s << kStripShift) : kStripCols;
+    return s * strip_rows(T, kStripCols) * kStripCols + (t + (c >> 1) + kRowShift) * nl + c;
 }
 __host__ __device__ __forceinline__ i64 boundary_entries(i64 T, i64 Up) {
-    return ((Up - 1) >> 6) * (T + kBndPad);
+    return ((Up - 1) >> kStripShift) * (T + kBndPad);
 }
 
-// What the gather pass leaves per lattice cell: one 16-byte store per compact row; each lattice
-// walk reads the 8-byte half of its number system.
-struct __attribute__((aligned(16))) LpCell {
+// What the gather pass leaves per lattice cell: two 8-byte records in two arrays of the strip
+// layout, the probabilities for the linear-domain walk and the logarithms for the log-domain walk
+// and the gradient fill.  Kept apart so that a lane of the lattice walk fetches what it needs of its
+// two columns with one 16-byte load, and a strip row of the walk touches no byte it does not use:
+// the walks are bound by what their memory instructions move through the CU's vector memory path
+// as much as by their arithmetic (widening the probabilities to fp64 in this pass, which saves the
+// walk four conversions a step and costs it one more 16-byte load, made every walk slower).
+struct LpCell {
     float p_blank;  // 2^l_blank
     float p_label;  // 2^l_label
     float l_blank;  // log2 P(blank | t,u)
     float l_label;  // log2 P(y[u] | t,u); 0 in the last column
+};
+struct LpStore {
+    float2* p;  // slot_cap  (P(blank), P(label))
+    float2* l;  // slot_cap  (log2 P(blank), log2 P(label))
+    struct Ref {
+        float2* p;
+        float2* l;
+        __device__ __forceinline__ void operator=(const LpCell& c) const {
+            *p = make_float2(c.p_blank, c.p_label);
+            *l = make_float2(c.l_blank, c.l_label);
+        }
+    };
+    __device__ __forceinline__ Ref operator[](i64 i) const { return Ref{p + i, l + i}; }
 };
 
 // Cost of a sequence from its two likelihoods, both as base-2 logarithms: fwd = alpha at the last
@@ -291,7 +316,7 @@ __device__ __forceinline__ int fetch_label(const RowInfo& ri, const int* __restr
     return lab;
 }
 
-// What the lattice walk consumes, one 16-byte record per cell (see LpCell): the (blank, label)
+// What the lattice walk consumes, two 8-byte records per cell (see LpCell, LpStore): the (blank, label)
 // log-probabilities as base-2 logarithms, floored so that -inf logits stay finite, and the same
 // two as plain probabilities for the scaled linear-domain walk.  A logarithm outside
 // [kLinMin, kLinMax] cannot be carried by that walk within one of its blocks (nor, as a

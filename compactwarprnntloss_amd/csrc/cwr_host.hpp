@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/cwarp_rnnt_hip.h"
+#include "cwr_device.hpp"
 
 namespace cwr {
 
@@ -40,7 +41,7 @@ struct Workspace {
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
     int* seqmode;   // N+1  per sequence: 0 = walked in the scaled linear domain; bit 0 = in the log domain
                     //      (gather's verdict), bits 1 / 2 = alpha / beta repeated in the log domain
-    LpCell* lp;     // slot_cap  gathered (blank, label) log-probabilities and probabilities
+    LpStore lp;     // 2 x slot_cap  gathered (blank, label) probabilities and log-probabilities
     double* alpha;  // slot_cap  log2(alpha), or alpha * 2^scale_a[block][column] (see seqmode)
     double* beta;   // slot_cap
     int* scale_a;   // slot_cap/16+1  per strip: exponent of each (16-step block, column) of the alpha walk

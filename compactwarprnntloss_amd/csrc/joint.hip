@@ -335,7 +335,7 @@ template <int ND> __device__ __forceinline__ void fwd_merge_halves(FwdRows<ND>& 
 }
 
 struct FwdOut {
-    LpCell* lp;
+    LpStore lp;
     float* lse;
     int2* rowinfo;
     float2* grads_skipped;

@@ -6,10 +6,11 @@
 //   cwarp_cuda_rnnt_kernel.cu:275-367         -> k_fill     (fill_grad_blank/label, fill_cost)
 //   cwarp_cuda_rnnt_kernel.cu:575             -> k_cost_from_beta
 //
-// Lattice walk: one wave owns a strip of 64 label positions of one sequence and walks it along
-// the anti-diagonals; at step q lane l holds cell (t = q - l, u = 64 s + l).  The neighbour in u
-// is the adjacent lane (one DPP wave shift), the neighbour in t is the lane's own previous value,
-// so a step needs no barrier.  A lone wave issues one instruction every four to five cycles
+// Lattice walk: one wave owns a strip of 128 label positions of one sequence, two per lane, and
+// walks it along skewed diagonals; at step q lane l holds the cells (t = q - l, u = 128 s + 2l) and
+// (t, u + 1).  The neighbour in u of the lane's first column is the adjacent lane (one DPP wave
+// shift), that of its second column the lane itself, the neighbour in t is the lane's own previous
+// value, so a step needs no barrier.  A lone wave issues one instruction every four to five cycles
 // whatever its kind, so the step is written for the smallest instruction count:
 //   - the strip layout (see lattice_slot) makes every step's access one row at a constant pitch:
 //     buffer instructions with a per-lane constant offset and a scalar row offset, no address
@@ -18,6 +19,8 @@
 //     recursion keeps them at the "no path" marker by itself (see below);
 //   - the normal number system is the scaled linear domain (one fp64 add and two multiplies per
 //     cell); base-2 logarithms on the v_exp_f32 / v_log_f32 units are the fallback.
+#include <atomic>
+
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
@@ -27,7 +30,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
 constexpr int kOob = (int)0x80000000;  // per-lane offset that every buffer range check rejects
-constexpr int kMaxFrames = 1 << 20;    // keeps a strip below the 2 GiB a buffer descriptor spans
+constexpr int kMaxFrames = 1 << 19;    // keeps a strip below the 2 GiB a buffer descriptor spans
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, i64 bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
@@ -46,9 +49,13 @@ __device__ __forceinline__ void buf_store_d(__amdgpu_buffer_rsrc_t r, int voff, 
     v.y = __double2hiint(x);
     __builtin_amdgcn_raw_buffer_store_b64(v, r, voff, soff, 0);
 }
-__device__ __forceinline__ void buf_store_zero16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    v4i z = {0, 0, 0, 0};
-    __builtin_amdgcn_raw_buffer_store_b128(z, r, voff, soff, 0);
+__device__ __forceinline__ void buf_store_d2(__amdgpu_buffer_rsrc_t r, int voff, int soff, double x, double y) {
+    v4i v = {__double2loint(x), __double2hiint(x), __double2loint(y), __double2hiint(y)};
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, 0);
+}
+__device__ __forceinline__ void buf_store_zero8(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    v2i z = {0, 0};
+    __builtin_amdgcn_raw_buffer_store_b64(z, r, voff, soff, 0);
 }
 __device__ __forceinline__ float buf_load_f(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     return __int_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
@@ -57,14 +64,17 @@ __device__ __forceinline__ void buf_store_i32(__amdgpu_buffer_rsrc_t r, int voff
     __builtin_amdgcn_raw_buffer_store_b32(x, r, voff, soff, 0);
 }
 
-// k_fill works in chunks of kFillRows rows of one strip (its rows that hold cells: T + nl - 1 of
-// them); a sequence's chunks are numbered strip by strip.  Few rows per chunk: many short waves,
-// whose dependent loads (chunk -> sequence -> lattice values -> their scales) overlap across waves.
-constexpr int kFillRows = 4;
-__host__ __device__ __forceinline__ i64 strip_chunks(i64 T, i64 nl) { return (T + nl - 1 + kFillRows - 1) / kFillRows; }
+// k_fill works in chunks of kFillSlots consecutive slots of the cell rows of one strip (its rows
+// that hold cells: T + lanes - 1 of them, nl slots each); a sequence's chunks are numbered strip by
+// strip.  Small chunks: many short waves, whose dependent loads (chunk -> sequence -> lattice
+// values -> their scales) overlap across waves.
+constexpr int kFillSlots = 256;
+__host__ __device__ __forceinline__ i64 strip_chunks(i64 T, i64 nl) {
+    return ((T + strip_lanes(nl) - 1) * nl + kFillSlots - 1) / kFillSlots;
+}
 __host__ __device__ __forceinline__ i64 fill_chunks(i64 T, i64 Up) {
-    const i64 full = (Up - 1) >> 6;
-    return full * strip_chunks(T, 64) + strip_chunks(T, Up - (full << 6));
+    const i64 full = (Up - 1) >> kStripShift;
+    return full * strip_chunks(T, kStripCols) + strip_chunks(T, Up - (full << kStripShift));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -179,22 +189,28 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 // ---------------------------------------------------------------------------------------------
 // lattice
 // ---------------------------------------------------------------------------------------------
-// Walk one strip of nl columns and T frames, Q = T+nl-1 steps; step k handles row q = k (alpha)
-// or q = Q-1-k (beta) of the strip.  With a = value of the cell, B / L its blank / label log-prob:
-//   alpha: a = own (+) nbr;  own' = a (x) B(t,u);    nbr' = a (x) L(t,u)     -> cells (t+1,u), (t,u+1)
-//   beta : a = own (+) nbr;  own' = a (x) B(t-1,u);  nbr' = a (x) L(t,u-1)   -> cells (t-1,u), (t,u-1)
+// Walk one strip of nl columns (two per lane: lane j holds columns 2j and 2j+1 of the strip) and T
+// frames.  At step k of Q = T + lanes - 1 the wave handles strip row q = k (alpha) or q = Q-1-k
+// (beta): lane j the two cells of frame t = q - j.  With a = value of a cell, B / L its blank /
+// label probability, and (c0, c1) the lane's columns:
+//   alpha: a0 = own0 (+) nbr;          own0' = a0 (x) B(t,c0);    p = a0 (x) L(t,c0)
+//          a1 = own1 (+) p;            own1' = a1 (x) B(t,c1);    nbr' = a1 (x) L(t,c1)    -> lane j+1
+//   beta : a1 = own1 (+) nbr;          own1' = a1 (x) B(t-1,c1);  p = a1 (x) L(t,c0)
+//          a0 = own0 (+) p;            own0' = a0 (x) B(t-1,c0);  nbr' = a0 (x) L(t,c0-1)  -> lane j-1
 // i.e. every cell applies the transition INTO its successor, so that the only operations between
-// receiving the neighbour's value and handing one's own on are those of (+) itself (beta fetches
-// L(t,u-1) from the lane on its left one step ahead of time).
+// receiving the neighbour's value and handing one's own on are the two (+) and two (x) of the
+// lane's pair (beta fetches L(t,c0-1) from the lane on its left one step ahead of time).  Two
+// columns per lane: a diagonal step serves twice the label positions for one cross-lane move, one
+// store and one set of loop bookkeeping, and a sequence of up to 512 labels keeps every wave of its
+// workgroup on a SIMD of its own.
 //
 // Two number systems implement ((+), (x)):
-//   linear  values are probabilities times 2^C, C an integer kept per block of kPF steps; (+) is
-//           an fp64 add and (x) an fp64 multiply, so the dependent chain of a step is
-//           DPP shift -> add -> multiply.  At the start of every block the wave takes the largest
-//           exponent among its lanes (and among the values about to come in from the previous
-//           strip), renormalises to 2^kLinTarget and records C for k_fill.  The gather pass has
-//           checked that no log-prob of the sequence can push a value out of the fp64 range
-//           within one block (kLinMin, kLinMax).
+//   linear  values are probabilities times 2^C, C an integer kept per lane and block of kPF steps;
+//           (+) is an fp64 add and (x) an fp64 multiply.  At the start of every block every lane
+//           renews its scale so that the largest magnitude it can meet during the block sits at
+//           2^kLinTarget, and records C for k_fill.  The gather pass has checked that no log-prob
+//           of the sequence can push a value out of the fp64 range within one block (kLinMin,
+//           kLinMax).
 //   log     values are base-2 logarithms in fp64, (+) is max + log2(1 + 2^-|d|) on the fp32
 //           exp2/log2 units, (x) an add.  Used for the sequences the gather pass marked (extreme
 //           log-probs) and for those with more strips than waves.
@@ -205,13 +221,13 @@ int launch_offsets(const int* lx, const int* ly, i64 N, i64 R, i64 max_u, i64 sl
 //   - the start cell is produced by seeding its lane's `own`;
 //   - after its last cell a lane computes junk that no lane with a cell reads any more, and
 //     stores it into padding slots;
-//   - lanes >= nl use an offset every buffer range check rejects (loads give 0, stores vanish).
+//   - columns >= nl use an offset every buffer range check rejects (loads give 0, stores vanish).
 //
 // A strip hands the values of its edge column to the next strip through a boundary stream
-// indexed by the producer's step; the receiving edge lane takes the value in as the `old` operand
-// of the DPP shift, so it lands in the lane that has no neighbour.  The stream is either a ring in
-// LDS (strips walked concurrently by one wave each) or, for the log walk of very long label
-// sequences, a span of global memory (strips walked one after the other by one wave).
+// indexed by the producer's step; the receiving edge lane adds the value to the `own` of its edge
+// column.  The stream is either a ring in LDS (strips walked concurrently by one wave each) or, for
+// the log walk of very long label sequences, a span of global memory (strips walked one after the
+// other by one wave).
 constexpr int kRing = 256;             // entries of an LDS boundary ring (a multiple of kPF)
 constexpr int kSpinLimit = 1 << 22;    // polls after which a waiting wave gives up
 constexpr int kNoExp = -(1 << 20);     // "exponent" of zero
@@ -261,31 +277,58 @@ __device__ __forceinline__ void keep_order() { __atomic_signal_fence(__ATOMIC_SE
 // one trip earlier: the compiler derives ONE wait count per consuming instruction, the strictest
 // over all ways of reaching it, and on the way in from the initial fill the registers consumed
 // first may have been loaded last.  Without this that wait (all loads but one) would be paid on
-// every trip; with it only the loop's own distance (kPF loads) counts.
+// every trip; with it only the loop's own distance (kPF steps of loads) counts.
 __device__ __forceinline__ void settle_loads() {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), other counters untouched
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// Both walks share one shape.  A ring of kPF registers holds the gathered records of the next
-// kPF steps; step j issues the load that refills ring[j] and prepares the NEXT step's two
-// transition terms from ring[j+1], so a ring register is dead when its refill is issued (the
-// register allocator then keeps every ring entry in place: no copies of registers with a load in
-// flight, which would make the wave wait for memory at every block) and the conversions stay off
+// Both walks share one shape.  Two rings of kPF registers hold the gathered records of the lane's
+// two columns for the next kPF steps; step j issues the loads that refill entry j and prepares the
+// NEXT step's transition terms from entry j+1, so a ring register is dead when its refill is issued
+// (the register allocator then keeps every ring entry in place: no copies of registers with a load
+// in flight, which would make the wave wait for memory at every block) and the conversions stay off
 // the dependent chain.  The values that enter from the previous strip are prepared once per block
 // by lanes 0..kPF-1 (lane j: the value entering at step k0+j) and picked per step with a readlane.
+
+// Per-lane byte offsets of a lane's two columns into a row of records of `bytes` each; a column the
+// strip does not have gets the offset every range check rejects.
+struct LaneCols {
+    int c0, c1;
+};
+__device__ __forceinline__ LaneCols lane_cols(int lane, int nl, int bytes) {
+    LaneCols lc;
+    lc.c0 = 2 * lane < nl ? 2 * lane * bytes : kOob;
+    lc.c1 = 2 * lane + 1 < nl ? (2 * lane + 1) * bytes : kOob;
+    return lc;
+}
+
+// The records of a lane's two columns in one row: one 16-byte load, or two 8-byte loads when the
+// strip's last lane has one column only (the missing one then reads as zeros).
+template <bool ODD>
+__device__ __forceinline__ float4 load_pair(__amdgpu_buffer_rsrc_t r, const LaneCols v, int soff) {
+    if (ODD) {
+        const float2 a = buf_load_f2(r, v.c0, soff), b = buf_load_f2(r, v.c1, soff);
+        return make_float4(a.x, a.y, b.x, b.y);
+    }
+    const v4i x = __builtin_amdgcn_raw_buffer_load_b128(r, v.c0, soff, 0);
+    return make_float4(__int_as_float(x.x), __int_as_float(x.y), __int_as_float(x.z), __int_as_float(x.w));
+}
 
 // Zeroes the triangle of padding records a direction reads before a lane's first cell.  A zero
 // record is "probability 0" for the linear walk and "log-prob 0" for the log walk; both keep a
 // lane that holds "no path" there (junk in those records could be a NaN, which nothing survives).
 template <bool BETA>
 __device__ __forceinline__ void clear_leading(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
-    const int p16 = nl * 16;
+    const int p8 = nl * 8;
+    const int nlane = (int)strip_lanes(nl);
+    const LaneCols vc = lane_cols(lane, nl, 8);
 #pragma unroll 4
-    for (int j = 0; j < nl - 1; ++j) {
+    for (int j = 0; j < nlane - 1; ++j) {
         const int row = (BETA ? T + j : j) + kRowShift;
-        const bool mine = BETA ? lane <= j : (lane > j && lane < nl);
-        buf_store_zero16(r_cell, mine ? lane * 16 : kOob, row * p16);
+        const bool mine = BETA ? lane <= j : lane > j;
+        buf_store_zero8(r_cell, mine ? vc.c0 : kOob, row * p8);
+        buf_store_zero8(r_cell, mine ? vc.c1 : kOob, row * p8);
     }
     __threadfence_block();
 }
@@ -296,59 +339,74 @@ __device__ __forceinline__ void clear_leading(__amdgpu_buffer_rsrc_t r_cell, int
 // Both directions of a sequence clear the same records; nothing else is ever written to them.
 template <bool BETA>
 __device__ __forceinline__ void clear_around(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
-    const int p16 = nl * 16;
-    const int Q = T + nl - 1;
-    const int vo = lane < nl ? lane * 16 : kOob;
+    const int p8 = nl * 8;
+    const int nlane = (int)strip_lanes(nl);
+    const int Q = T + nlane - 1;
+    const LaneCols vc = lane_cols(lane, nl, 8);
     // row j of the cells' bounding box: lanes > j have not started; in row T+j lanes <= j have
     // finished; one store covers both (the per-lane offset picks the row)
 #pragma unroll 4
-    for (int j = 0; j < nl - 1; ++j)
-        buf_store_zero16(r_cell, lane < nl ? lane * 16 + (lane > j ? 0 : T * p16) : kOob, (j + kRowShift) * p16);
+    for (int j = 0; j < nlane - 1; ++j) {
+        const int shift = lane > j ? 0 : T * p8;
+        buf_store_zero8(r_cell, vc.c0 == kOob ? kOob : vc.c0 + shift, (j + kRowShift) * p8);
+        buf_store_zero8(r_cell, vc.c1 == kOob ? kOob : vc.c1 + shift, (j + kRowShift) * p8);
+    }
 #pragma unroll 4
-    for (int j = 1; j <= kPF; ++j)
-        buf_store_zero16(r_cell, vo, (BETA ? kRowShift - j : Q - 1 + j + kRowShift) * p16);
+    for (int j = 1; j <= kPF; ++j) {
+        buf_store_zero8(r_cell, vc.c0, (BETA ? kRowShift - j : Q - 1 + j + kRowShift) * p8);
+        buf_store_zero8(r_cell, vc.c1, (BETA ? kRowShift - j : Q - 1 + j + kRowShift) * p8);
+    }
     __threadfence_block();
 }
 
-// Range check of the linear walk.  Every kCheckEvery-th step all cell values must lie inside
-// [2^kLowExp, 2^kHighExp) at their lane's scale; otherwise the walk reports the direction as
-// unsafe and it is walked again in the log domain.  In between, a value descends from checked ones
-// through at most kCheckEvery products with factors in [2^kLinMin, 2^(kLinMax+1)], so inside the
-// bounds no product can leave the normal fp64 range (-600 - 4*100 > -1022, 980 + 4*9 < 1023): the
-// results are then exact up to rounding, whatever the spread of magnitudes across the lattice.
-constexpr int kCheckEvery = 4;
+// Range check of the linear walk.  All cell values must lie inside [2^kLowExp, 2^kHighExp) at their
+// lane's scale, the lower bound looked at every kCheckLow-th step and the upper one every
+// kCheckHigh-th; otherwise the walk reports the direction as unsafe and it is walked again in the
+// log domain.  In between, a value descends from checked ones through at most two products per
+// step (two columns per lane) with factors in [2^kLinMin, 2^(kLinMax+1)], so inside the bounds no
+// product can leave the normal fp64 range (-600 - 4*100 > -1022, 1000 + 8*2 < 1023): the results
+// are then exact up to rounding, whatever the spread of magnitudes across the lattice.  The lower
+// bound is the one real data comes near (a lane's scale follows the largest of what it holds and
+// hands on, and a cell whose blank is improbable holds 2^-90 of what it hands on), hence its
+// closer watch.
+constexpr int kCheckLow = 2;
+constexpr int kCheckHigh = 4;
 constexpr int kLowExp = -600;
-constexpr int kHighExp = 980;
+constexpr int kHighExp = 1000;
 constexpr unsigned kLowHigh = (unsigned)(1023 + kLowExp) << 20;    // high word of 2^kLowExp
 constexpr unsigned kHighHigh = (unsigned)(1023 + kHighExp) << 20;  // high word of 2^kHighExp
 
 // ---- scaled linear-domain walk (strips concurrent, LDS rings) -------------------------------
-// Every LANE carries its own scale: the values of column u are probabilities times 2^C[u], with
-// C[u] renewed at the start of every block of kPF steps so that the larger of the lane's own value
+// Every LANE carries its own scale: the values of its two columns are probabilities times 2^C, with
+// C renewed at the start of every block of kPF steps so that the largest of the lane's own values
 // and of what its neighbour is about to hand over sits at 2^kLinTarget.  A value arriving from the
 // neighbouring lane is brought to the lane's scale by one v_ldexp_f64 with the (block-constant)
-// difference of the two scales.  Like a logarithm, this loses nothing across columns, however far
+// difference of the two scales.  Like a logarithm, this loses nothing across lanes, however far
 // apart their magnitudes are: the only thing that can underflow is a summand that is negligible
-// next to the other summand of the SAME cell.  Within a block a lane's value can still drift out
-// of the fp64 range (a run of extreme factors, or a much larger magnitude arriving from several
-// columns away), which the range check catches.  Returns false when the check failed.
-template <bool BETA, bool HAS_IN, bool HAS_OUT>
-__device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const bool seed, const int in_shift,
-                                                const int out_shift, const LpCell* lp_strip,
+// next to the other summand of the SAME cell, or one of a lane's two columns next to the other.
+// Within a block a lane's value can still drift out of the fp64 range (a run of extreme factors,
+// or a much larger magnitude arriving from several columns away), which the range check catches.
+// ODD: the strip's last lane has one column only (nl odd); the pair is then stored as two 8-byte
+// values, the missing one at the rejected offset.  seed_col: column of this strip that holds the
+// start cell of the walk, or -1.  Returns false when the check failed.
+template <bool BETA, bool HAS_IN, bool HAS_OUT, bool ODD>
+__device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const int seed_col, const int in_shift,
+                                                const int out_shift, const float2* lp_strip,
                                                 double* out_strip, int* scale_strip, const Ring rin,
                                                 const Ring rout, const WaitCtl wc) {
     const int lane = threadIdx.x & 63;
-    const int Q = T + nl - 1;
+    const int nlane = (int)strip_lanes(nl);
+    const int Q = T + nlane - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    const int p16 = nl * 16, p8 = nl * 8, p4 = nl * 4;
-    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
+    const int p8 = nl * 8, p4 = nlane * 4;
+    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * p4);
-    const int vo_p = lane < nl ? lane * 16 : kOob;  // the two probabilities of a record
-    const int vo = lane < nl ? lane * 8 : kOob;
-    const int vo_sc = lane < nl ? lane * 4 : kOob;
-    constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 64 wide
+    const LaneCols vo = lane_cols(lane, nl, 8);  // a lane's two columns in a row of 8-byte records
+    const LaneCols vp = vo;
+    const int vo_sc = lane < nlane ? lane * 4 : kOob;
+    constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 128 wide
     constexpr int out_lane = BETA ? 0 : 63;
     double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
     constexpr int dq = BETA ? -1 : 1;
@@ -358,32 +416,44 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     const int row0 = (BETA ? Q - 1 : 0) + kRowShift;  // row of step 0
     int qi = row0;                                    // row of the current step
     int mi = BETA ? row0 - 1 : row0;                  // row that holds the current step's multipliers
-    float2 ring[kPF];                                 // (blank, label) probabilities, rows mi .. mi+dq*(kPF-1)
+    float4 ring[kPF];  // (blank, label) probabilities of the two columns, rows mi .. mi+dq*(kPF-1)
 #pragma unroll
-    for (int j = 0; j < kPF; ++j) ring[j] = buf_load_f2(r_cell, vo_p, (mi + dq * j) * p16);
+    for (int j = 0; j < kPF; ++j) ring[j] = load_pair<ODD>(r_cell, vp, (mi + dq * j) * p8);
     int C = kLinTarget;  // this lane's scale exponent
     int d = 0;           // C minus the scale exponent of the lane the neighbour values come from
     // alpha[0][0] = 1; beta[T-1][U] = blank probability of that cell
-    double own = 0.0;
-    if (BETA) {
-        const float pb = buf_load_f(r_cell, seed ? lane * 16 : kOob, row0 * p16);
-        own = seed ? __builtin_ldexp((double)pb, kLinTarget) : 0.0;
-    } else {
-        own = seed ? __builtin_ldexp(1.0, kLinTarget) : 0.0;
+    double own0 = 0.0, own1 = 0.0;
+    float l_row0 = 0.f;  // beta: L(t,c0) of the row of step 0
+    {
+        const bool seed0 = seed_col == 2 * lane, seed1 = seed_col == 2 * lane + 1;
+        if (BETA) {
+            const float pb = buf_load_f(r_cell, (seed0 || seed1) ? seed_col * 8 : kOob, row0 * p8);
+            l_row0 = buf_load_f(r_cell, vp.c0 == kOob ? kOob : vp.c0 + 4, row0 * p8);
+            const double sv = __builtin_ldexp((double)pb, kLinTarget);
+            own0 = seed0 ? sv : 0.0;
+            own1 = seed1 ? sv : 0.0;
+        } else {
+            own0 = seed0 ? __builtin_ldexp(1.0, kLinTarget) : 0.0;
+        }
     }
     double pass = 0.0;
     double nbr = 0.0;  // the edge lane has no neighbour: it keeps "no path" here for good
-    // alpha applies its own cell's probabilities; beta B(t-1,u) and L(t,u-1), the latter from the
-    // lane on its left (lane 0 gets 0: nobody reads its `pass`)
-    double mul_own = (double)ring[0].x;
-    double mul_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].y) : ring[0].y);
+    // alpha applies its own cells' probabilities: (B0, L0, B1, L1) of the row.  beta applies
+    // B(t-1,c0), B(t-1,c1) of the row before, L(t,c0) of the row itself (kept from the step before)
+    // and L(t,c0-1), which is the second label probability the lane on its left holds for the row
+    // before (lane 0 gets 0: nobody reads its `pass`)
+    double mB0 = (double)ring[0].x, mB1 = (double)ring[0].z;
+    double mL0 = BETA ? (double)l_row0 : (double)ring[0].y;
+    double mL1 = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].w) : ring[0].w);
+    double mL0_next = BETA ? (double)ring[0].y : 0.0;  // beta: L(t-1,c0), for the step after this one
     const double in_mask = lane == in_lane ? 1.0 : 0.0;
     unsigned lo_seen = 0xffffffffu, hi_seen = 0u;  // extremes of the cell values' high words (zero excluded)
     // beta hands on plain beta(t,u+1); the receiving edge column applies its own L(t,u), fetched
     // one block ahead by the lanes that prepare the incoming entries
     const int jl = lane & (kPF - 1);
+    constexpr int edge_off = (kStripCols - 1) * 8 + 4;
     float edge = 0.f;
-    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p16 + 63 * 16 + 4, 0);
+    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p8 + edge_off, 0);
     settle_loads();
     int k0 = 0;
     for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
@@ -413,17 +483,18 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         keep_order();
         // Renew the scales.  True magnitude (binary exponent minus scale) of what the lane holds,
         // of what it will hand over and of what its neighbour will hand over next:
-        const int t_own = own != 0.0 ? __builtin_amdgcn_frexp_exp(own) - C : kNoExp;
+        const int t_own0 = own0 != 0.0 ? __builtin_amdgcn_frexp_exp(own0) - C : kNoExp;
+        const int t_own1 = own1 != 0.0 ? __builtin_amdgcn_frexp_exp(own1) - C : kNoExp;
         const int t_pass = pass != 0.0 ? __builtin_amdgcn_frexp_exp(pass) - C : kNoExp;
-        int t = max(max(t_own, t_pass),
-                    BETA ? dpp_i32<DPP_WAVE_SHL1>(kDppMin, t_pass) : dpp_i32<DPP_WAVE_SHR1>(kDppMin, t_pass));
+        int t = max(max(t_own0, t_own1),
+                    max(t_pass, BETA ? dpp_i32<DPP_WAVE_SHL1>(kDppMin, t_pass) : dpp_i32<DPP_WAVE_SHR1>(kDppMin, t_pass)));
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
             double ev = en_first;
             if (BETA) {
                 ev *= (double)edge;
-                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p16 + 63 * 16 + 4, 0);
+                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p8 + edge_off, 0);
             }
             // entry k0+j feeds frame k0+j of the edge column: beyond the last frame it is junk
             const bool ok = k0 + jl < T && ev != 0.0;
@@ -439,7 +510,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         }
         // Whatever reaches a lane during this block was, at its start, in one of the kPF lanes the
         // values come from (or enters through the edge lane, counted above): take the largest
-        // magnitude over that window, so that nothing arriving can exceed 2^(kLinTarget + kPF*
+        // magnitude over that window, so that nothing arriving can exceed 2^(kLinTarget + 2*kPF*
         // (kLinMax+1)).  Window used: the lanes before it in its row of 16 and the whole row before.
         if (BETA) {
             t = max(t, dpp_i32<DPP_ROW_SHL + 1>(kDppMin, t));
@@ -463,38 +534,65 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         const bool empty = t <= kNoExp / 2;
         int Cn = empty ? C : kLinTarget - t;
         // a lane that holds nothing yet takes the scale of the lane that started last: whatever
-        // reaches it during this block has come from there, through at most kPF products
-        const int started = BETA ? nl - k0 : k0 - 1;
-        const int last = started < 0 ? 0 : (started > nl - 1 ? nl - 1 : started);
+        // reaches it during this block has come from there, through at most 2*kPF products
+        const int started = BETA ? nlane - k0 : k0 - 1;
+        const int last = started < 0 ? 0 : (started > nlane - 1 ? nlane - 1 : started);
         const int Cref = __builtin_amdgcn_readlane(Cn, last);
         Cn = empty ? Cref : Cn;
-        own = __builtin_ldexp(own, Cn - C);
+        own0 = __builtin_ldexp(own0, Cn - C);
+        own1 = __builtin_ldexp(own1, Cn - C);
         pass = __builtin_ldexp(pass, Cn - C);
         C = Cn;
         d = C - (BETA ? dpp_i32<DPP_WAVE_SHL1>(C, C) : dpp_i32<DPP_WAVE_SHR1>(C, C));
-        if (lane >= nl) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
+        if (lane >= nlane) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
         if (HAS_IN) e_lane = __builtin_ldexp(e_lane, __builtin_amdgcn_readlane(C, in_lane) - cp);
         buf_store_i32(r_sc, vo_sc, __builtin_amdgcn_readfirstlane(blk * p4), C);  // wave-uniform, and said so
         if (HAS_OUT) rout.scales[(k0 / kPF) & (kRing / kPF - 1)] = __builtin_amdgcn_readlane(C, out_lane);
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
-            const float2 cn = buf_load_f2(r_cell, vo_p, (mi + dq * kPF) * p16);
-            double o = own;
-            if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own);
+            const float4 cn = load_pair<ODD>(r_cell, vp, (mi + dq * kPF) * p8);
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(nbr, pass) : dpp_f64<DPP_WAVE_SHR1>(nbr, pass);
-            const double a = o + __builtin_ldexp(nbr, d);
-            own = a * mul_own;
-            pass = a * mul_pass;
-            if (j % kCheckEvery == 0) {
-                const unsigned h = (unsigned)__double2hiint(a);
-                lo_seen = min(lo_seen, h - 1u);  // zero wraps to the top and drops out
-                hi_seen = max(hi_seen, h);
+            double a0, a1;
+            if (BETA) {
+                double o = own1;
+                if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own1);
+                a1 = o + __builtin_ldexp(nbr, d);
+                own1 = a1 * mB1;
+                a0 = own0 + a1 * mL0;
+                own0 = a0 * mB0;
+                pass = a0 * mL1;
+            } else {
+                double o = own0;
+                if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own0);
+                a0 = o + __builtin_ldexp(nbr, d);
+                own0 = a0 * mB0;
+                a1 = own1 + a0 * mL0;
+                own1 = a1 * mB1;
+                pass = a1 * mL1;
             }
-            buf_store_d(r_out, vo, qi * p8, a);
-            if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = BETA ? a : pass;
-            const float2 nx = ring[(j + 1) % kPF];
-            mul_own = (double)nx.x;
-            mul_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.y) : nx.y);
+            if (j % kCheckLow == 0) {
+                const unsigned h0 = (unsigned)__double2hiint(a0), h1 = (unsigned)__double2hiint(a1);
+                lo_seen = min(lo_seen, min(h0 - 1u, h1 - 1u));  // zero wraps to the top and drops out
+                if (j % kCheckHigh == 0) hi_seen = max(hi_seen, max(h0, h1));
+            }
+            if (ODD) {
+                buf_store_d(r_out, vo.c0, qi * p8, a0);
+                buf_store_d(r_out, vo.c1, qi * p8, a1);
+            } else {
+                buf_store_d2(r_out, vo.c0, qi * p8, a0, a1);
+            }
+            if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = BETA ? a0 : pass;
+            const float4 nx = ring[(j + 1) % kPF];
+            mB0 = (double)nx.x;
+            mB1 = (double)nx.z;
+            if (BETA) {
+                mL0 = mL0_next;
+                mL0_next = (double)nx.y;
+                mL1 = (double)dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.w);
+            } else {
+                mL0 = (double)nx.y;
+                mL1 = (double)nx.w;
+            }
             ring[j] = cn;
             qi += dq;
             mi += dq;
@@ -503,10 +601,14 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             __builtin_amdgcn_sched_barrier(0);
         }
         keep_order();
-        const int done = blk + 1 == nblocks ? 0x7fffffff : k0 + kPF;
-        if (HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        // no "last block" case in here: a select on the block count has been seen compiled into a
+        // scalar select that reads a condition code nobody set (the count lived in a vector register)
+        if (HAS_OUT) __hip_atomic_store(rout.produced, k0 + kPF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (HAS_IN) __hip_atomic_store(rin.consumed, k0 + kPF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    // done: whatever the neighbours still wait for will not come from here (or is not needed here)
+    if (HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     return __ballot(lo_seen < kLowHigh - 1u || hi_seen >= kHighHigh) == 0;
 }
 
@@ -514,22 +616,39 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
 // CONC: strips concurrent, boundary values through the LDS rings; otherwise one wave walks the
 // strips in turn and the boundary values travel through a stream in global memory, which the
 // lanes that prepare the incoming entries read one block ahead.
+//
+// log2(2^x + 2^y) = max + log2(1 + 2^-|x-y|): the form of cwarp_cuda_rnnt_kernel.cu:22-29 in
+// base 2; the running values are fp64, the correction term (at most 1) comes from the fp32
+// exp2 / log2 units.
+struct Lse2 {
+    double mx, l;  // the sum is mx + l
+};
+__device__ __forceinline__ Lse2 lse2(double x, double y) {
+    Lse2 r;
+    r.mx = fmax(x, y);
+    const float d = (float)(x - y);
+    r.l = (double)fast_log2(1.0f + fast_exp2(-fabsf(d)));
+    return r;
+}
+
 template <bool BETA, bool HAS_IN, bool HAS_OUT, bool CONC>
-__device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const bool seed, const int in_shift,
-                                                const int out_shift, const LpCell* lp_strip,
+__device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const int seed_col, const int in_shift,
+                                                const int out_shift, const float2* lp_strip,
                                                 double* out_strip, const double* bnd_in, double* bnd_out,
                                                 const Ring rin, const Ring rout, const WaitCtl wc) {
     const int lane = threadIdx.x & 63;
-    const int Q = T + nl - 1;
+    const int nlane = (int)strip_lanes(nl);
+    const int Q = T + nlane - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    const int p16 = nl * 16, p8 = nl * 8;
-    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p16);
+    const int p8 = nl * 8;
+    const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, (HAS_IN && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
     const __amdgpu_buffer_rsrc_t r_bo = make_rsrc(bnd_out, (HAS_OUT && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
-    const int vo_l = lane < nl ? lane * 16 + 8 : kOob;  // the two logarithms of a record
-    const int vo = lane < nl ? lane * 8 : kOob;
+    const LaneCols vo = lane_cols(lane, nl, 8);  // a lane's two columns in a row of 8-byte records
+    const LaneCols vl = vo;
+    constexpr int in_lane = BETA ? 63 : 0;
     constexpr int out_lane = BETA ? 0 : 63;
     const int vo_bo = lane == out_lane ? 0 : kOob;
     double* ring_out = rout.slots + (lane == out_lane ? 0 : kRing + lane);
@@ -540,25 +659,37 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     const int row0 = (BETA ? Q - 1 : 0) + kRowShift;
     int qi = row0;
     int mi = BETA ? row0 - 1 : row0;
-    float2 ring[kPF];  // (blank, label) logarithms, rows mi .. mi+dq*(kPF-1)
+    float2 ring0[kPF], ring1[kPF];  // (blank, label) logarithms, rows mi .. mi+dq*(kPF-1)
 #pragma unroll
-    for (int j = 0; j < kPF; ++j) ring[j] = buf_load_f2(r_cell, vo_l, (mi + dq * j) * p16);
-    // alpha: own = log 1 in the seed lane; beta: own = B of the seed lane's first cell
-    double own = kNeg;
-    if (BETA) {
-        const float lb = buf_load_f(r_cell, seed ? lane * 16 + 8 : kOob, row0 * p16);
-        own = seed ? (double)lb : kNeg;
-    } else {
-        own = seed ? 0.0 : kNeg;
+    for (int j = 0; j < kPF; ++j) {
+        ring0[j] = buf_load_f2(r_cell, vl.c0, (mi + dq * j) * p8);
+        ring1[j] = buf_load_f2(r_cell, vl.c1, (mi + dq * j) * p8);
+    }
+    // alpha: own = log 1 in the seed column; beta: own = B of the seed cell
+    double own0 = kNeg, own1 = kNeg;
+    float l_row0 = 0.f;
+    {
+        const bool seed0 = seed_col == 2 * lane, seed1 = seed_col == 2 * lane + 1;
+        if (BETA) {
+            const float lb = buf_load_f(r_cell, (seed0 || seed1) ? seed_col * 8 : kOob, row0 * p8);
+            l_row0 = buf_load_f(r_cell, vl.c0 == kOob ? kOob : vl.c0 + 4, row0 * p8);
+            own0 = seed0 ? (double)lb : kNeg;
+            own1 = seed1 ? (double)lb : kNeg;
+        } else {
+            own0 = seed0 ? 0.0 : kNeg;
+        }
     }
     double pass = kNeg;
     double nbr = kNeg;
-    double add_own = (double)ring[0].x;
-    double add_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].y) : ring[0].y);
+    double aB0 = (double)ring0[0].x, aB1 = (double)ring1[0].x;
+    double aL0 = BETA ? (double)l_row0 : (double)ring0[0].y;
+    double aL1 = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring1[0].y) : ring1[0].y);
+    double aL0_next = BETA ? (double)ring0[0].y : 0.0;
     const int jl = lane & (kPF - 1);
+    constexpr int edge_off = (kStripCols - 1) * 8 + 4;
     float edge = 0.f;      // beta: L(t,u) of the edge column's own cells, one block ahead
     double e_next = kNeg;  // global stream: the entries of the next block
-    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p16 + 63 * 16 + 12, 0);
+    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p8 + edge_off, 0);
     if (HAS_IN && !CONC) e_next = buf_load_d(r_in, jl * 8, in_shift * 8);
     settle_loads();
     int k0 = 0;
@@ -580,63 +711,95 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
             }
             if (BETA) {
                 ev += (double)edge;
-                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p16 + 63 * 16 + 12, 0);
+                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p8 + edge_off, 0);
             }
             e_lane = k0 + jl < T ? ev : kNeg;  // beyond the last frame the entries are junk
         }
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
-            const float2 cn = buf_load_f2(r_cell, vo_l, (mi + dq * kPF) * p16);
+            const float2 cn0 = buf_load_f2(r_cell, vl.c0, (mi + dq * kPF) * p8);
+            const float2 cn1 = buf_load_f2(r_cell, vl.c1, (mi + dq * kPF) * p8);
+            // the edge lane has no neighbour: the entry from the previous strip takes that place
             const double old = HAS_IN ? readlane_f64(e_lane, j) : nbr;
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(old, pass) : dpp_f64<DPP_WAVE_SHR1>(old, pass);
-            // log2(2^own + 2^nbr) = max + log2(1 + 2^-|own-nbr|): the form of
-            // cwarp_cuda_rnnt_kernel.cu:22-29 in base 2; the running values are fp64, the correction
-            // term (at most 1) comes from the fp32 exp2 / log2 units
-            const double mx = fmax(own, nbr);
-            const float d = (float)(own - nbr);
-            const double l = (double)fast_log2(1.0f + fast_exp2(-fabsf(d)));
-            const double a = mx + l;
-            own = (mx + add_own) + l;
-            pass = (mx + add_pass) + l;
-            buf_store_d(r_out, vo, qi * p8, a);
+            double a0, a1;
+            if (BETA) {
+                const Lse2 s1 = lse2(own1, nbr);
+                a1 = s1.mx + s1.l;
+                own1 = (s1.mx + aB1) + s1.l;
+                const Lse2 s0 = lse2(own0, (s1.mx + aL0) + s1.l);
+                a0 = s0.mx + s0.l;
+                own0 = (s0.mx + aB0) + s0.l;
+                pass = (s0.mx + aL1) + s0.l;
+            } else {
+                const Lse2 s0 = lse2(own0, nbr);
+                a0 = s0.mx + s0.l;
+                own0 = (s0.mx + aB0) + s0.l;
+                const Lse2 s1 = lse2(own1, (s0.mx + aL0) + s0.l);
+                a1 = s1.mx + s1.l;
+                own1 = (s1.mx + aB1) + s1.l;
+                pass = (s1.mx + aL1) + s1.l;
+            }
+            buf_store_d(r_out, vo.c0, qi * p8, a0);
+            buf_store_d(r_out, vo.c1, qi * p8, a1);
             if (HAS_OUT) {
-                const double h = BETA ? a : pass;  // alpha hands on a + L(t,u); beta plain a
+                const double h = BETA ? a0 : pass;  // alpha hands on a + L(t,u); beta plain a
                 if (CONC) ring_out[(k0 + j) & (kRing - 1)] = h;
                 else buf_store_d(r_bo, vo_bo, (k0 + j) * 8, h);
             }
-            const float2 nx = ring[(j + 1) % kPF];
-            add_own = (double)nx.x;
-            add_pass = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.y) : nx.y);
-            ring[j] = cn;
+            const float2 nx0 = ring0[(j + 1) % kPF], nx1 = ring1[(j + 1) % kPF];
+            aB0 = (double)nx0.x;
+            aB1 = (double)nx1.x;
+            if (BETA) {
+                aL0 = aL0_next;
+                aL0_next = (double)nx0.y;
+                aL1 = (double)dpp_f32_or_zero<DPP_WAVE_SHR1>(nx1.y);
+            } else {
+                aL0 = (double)nx0.y;
+                aL1 = (double)nx1.y;
+            }
+            ring0[j] = cn0;
+            ring1[j] = cn1;
             qi += dq;
             mi += dq;
             __builtin_amdgcn_sched_barrier(0);
         }
         if (CONC) keep_order();
-        const int done = blk + 1 == nblocks ? 0x7fffffff : k0 + kPF;
-        if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, k0 + kPF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, k0 + kPF, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    if (CONC && HAS_OUT) __hip_atomic_store(rout.produced, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// A strip's width is odd only when it is the last of its sequence: the alpha walk then has no strip
+// to feed, the beta walk none that feeds it.
 template <bool BETA>
-__device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
-                                             int out_shift, const LpCell* lp, double* out, int* sc, Ring rin,
+__device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, int nl, int seed_col, int in_shift,
+                                             int out_shift, const float2* lp, double* out, int* sc, Ring rin,
                                              Ring rout, const WaitCtl status) {
-    if (has_in && has_out) return sweep_strip_lin<BETA, true, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    if (has_in) return sweep_strip_lin<BETA, true, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    if (has_out) return sweep_strip_lin<BETA, false, true>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    return sweep_strip_lin<BETA, false, false>(T, nl, seed, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (nl & 1) {
+        if (BETA) {
+            if (has_out) return sweep_strip_lin<BETA, false, true, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+            return sweep_strip_lin<BETA, false, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+        }
+        if (has_in) return sweep_strip_lin<BETA, true, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+        return sweep_strip_lin<BETA, false, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    }
+    if (has_in && has_out) return sweep_strip_lin<BETA, true, true, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_in) return sweep_strip_lin<BETA, true, false, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_out) return sweep_strip_lin<BETA, false, true, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    return sweep_strip_lin<BETA, false, false, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
 }
 
 template <bool BETA, bool CONC>
-__device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, int nl, bool seed, int in_shift,
-                                             int out_shift, const LpCell* lp, double* out, const double* bi,
+__device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, int nl, int seed_col, int in_shift,
+                                             int out_shift, const float2* lp, double* out, const double* bi,
                                              double* bo, Ring rin, Ring rout, const WaitCtl status) {
-    if (has_in && has_out) sweep_strip_log<BETA, true, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else if (has_in) sweep_strip_log<BETA, true, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else if (has_out) sweep_strip_log<BETA, false, true, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
-    else sweep_strip_log<BETA, false, false, CONC>(T, nl, seed, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    if (has_in && has_out) sweep_strip_log<BETA, true, true, CONC>(T, nl, seed_col, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_in) sweep_strip_log<BETA, true, false, CONC>(T, nl, seed_col, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else if (has_out) sweep_strip_log<BETA, false, true, CONC>(T, nl, seed_col, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
+    else sweep_strip_log<BETA, false, false, CONC>(T, nl, seed_col, in_shift, out_shift, lp, out, bi, bo, rin, rout, status);
 }
 
 // One workgroup per (sequence, direction), W waves.  A sequence of S <= W strips is walked by S
@@ -644,13 +807,18 @@ __device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, i
 // demands plus one block of kPF steps of slack; the boundary values travel through LDS rings
 // guarded by two progress counters per ring.  A wave only ever waits for the wave of the strip
 // before it (values) or after it (ring space), and the first strip waits for nobody, so the chain
-// always drains; every wait is bounded all the same.  Longer sequences (S > W) fall back to one
-// wave walking the strips in turn, in the log domain, with the streams in global memory.
+// always drains; every wait is bounded all the same.  Longer sequences (S > W, 1024 labels or more)
+// fall back to one wave walking the strips in turn, in the log domain, with the streams in global
+// memory.
 constexpr int kMaxWaves = 8;
 
-__global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
+// At most two waves of this kernel share a SIMD (eight waves per workgroup, one workgroup per CU is
+// all a batch ever needs), which lets a wave keep both prefetch rings and the walk's state in up to
+// 256 registers; at the default budget of 128 the register allocator rotates the rings through
+// copies that wait for loads in flight and a step takes twice as long.
+__global__ __launch_bounds__(kMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(1, 2))) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
-    const i64* __restrict__ bnd_off, int* seqmode, const LpCell* lp, double* alpha,
+    const i64* __restrict__ bnd_off, int* seqmode, const LpStore lp, double* alpha,
     double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int spin_limit,
     int* status_word) {
     __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
@@ -663,7 +831,6 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const int dir = beta_only ? 1 : (int)blockIdx.y;
     const int W = blockDim.x >> 6;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int lane = threadIdx.x & 63;
     if (threadIdx.x < kMaxWaves) {
         s_produced[threadIdx.x] = 0;
         s_consumed[threadIdx.x] = 0;
@@ -676,11 +843,11 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     if (pad < 0) return;
     const int T = lx[n], U = ly[n];
     const int Up = U + 1;
-    const int S = (Up + 63) >> 6;
-    const i64 full_strip = strip_rows(T, 64) * 64;
+    const int S = (int)strip_count(Up);
+    const i64 full_strip = strip_rows(T, kStripCols) * kStripCols;
     double* out = dir ? beta : alpha;
     int* scale = dir ? scale_b : scale_a;
-    const int nl_last = Up - ((S - 1) << 6);
+    const int nl_last = Up - ((S - 1) << kStripShift);
     Ring none;
     none.slots = nullptr; none.scales = nullptr; none.produced = nullptr; none.consumed = nullptr;
 
@@ -691,21 +858,22 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         const bool active = w < S;
         const int p = active ? w : 0;
         const int s = dir ? S - 1 - p : p;
-        const int nl = s == S - 1 ? nl_last : 64;
+        const int nl = s == S - 1 ? nl_last : kStripCols;
         const i64 base = pad + (i64)s * full_strip;
         const bool has_in = p > 0, has_out = p < S - 1;
         Ring rin = none, rout = none;
         if (has_in) { rin.slots = s_ring[p - 1]; rin.scales = s_scale[p - 1]; rin.produced = &s_produced[p - 1]; rin.consumed = &s_consumed[p - 1]; }
         if (has_out) { rout.slots = s_ring[p]; rout.scales = s_scale[p]; rout.produced = &s_produced[p]; rout.consumed = &s_consumed[p]; }
         // alpha: the feeding strip's edge lane 63 trails its first lane by 63 steps; beta: the
-        // feeding strip is s+1 and its edge lane 0 trails by its width - 1; likewise for the strip fed
-        const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
-        const int out_shift = dir ? nl - 1 : 63;
-        const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
+        // feeding strip is s+1 and its edge lane 0 trails by its lanes - 1; likewise for the strip fed
+        const int in_shift = dir ? (int)strip_lanes(s + 1 == S - 1 ? nl_last : kStripCols) - 1 : 63;
+        const int out_shift = dir ? (int)strip_lanes(nl) - 1 : 63;
+        // alpha starts in cell (0,0), beta in cell (T-1,U)
+        const int seed_col = dir ? (s == S - 1 ? nl - 1 : -1) : (s == 0 ? 0 : -1);
         if (!linear) {
             if (active) {
-                if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
-                else log_dispatch<true, true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, nullptr, nullptr, rin, rout, status);
+                if (dir == 0) log_dispatch<false, true>(has_in, has_out, T, nl, seed_col, in_shift, out_shift, lp.l + base, out + base, nullptr, nullptr, rin, rout, status);
+                else log_dispatch<true, true>(has_in, has_out, T, nl, seed_col, in_shift, out_shift, lp.l + base, out + base, nullptr, nullptr, rin, rout, status);
             }
             __syncthreads();
             // a hand-over that never came: the lattice is incomplete, the sequence's cost becomes NaN
@@ -715,10 +883,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         bool safe = true;
         if (active) {
             int* sc = scale + (base >> 4);
-            safe = dir == 0 ? lin_dispatch<false>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status)
-                            : lin_dispatch<true>(has_in, has_out, T, nl, seed, in_shift, out_shift, lp + base, out + base, sc, rin, rout, status);
+            safe = dir == 0 ? lin_dispatch<false>(has_in, has_out, T, nl, seed_col, in_shift, out_shift, lp.p + base, out + base, sc, rin, rout, status)
+                            : lin_dispatch<true>(has_in, has_out, T, nl, seed_col, in_shift, out_shift, lp.p + base, out + base, sc, rin, rout, status);
         }
-        if (!safe && lane == 0) s_unsafe = 1;
+        if (!safe && (threadIdx.x & 63) == 0) s_unsafe = 1;
         __syncthreads();
         if (s_abort != 0) {
             if (threadIdx.x == 0) raise_flag(&seqmode[n], kSeqPoisoned);
@@ -727,7 +895,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
         if (s_unsafe == 0 || w != 0) return;
         // Some strip of this direction left the range the linear walk is exact in: wave 0 walks
         // the whole direction again, strip by strip, in the log domain (below).
-        if (lane == 0) atomicOr(&seqmode[n], dir ? 4 : 2);
+        if (threadIdx.x == 0) atomicOr(&seqmode[n], dir ? 4 : 2);
     }
 
     if (w != 0) return;
@@ -735,16 +903,16 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
     const i64 bstride = (i64)T + kBndPad;
     for (int p = 0; p < S; ++p) {
         const int s = dir ? S - 1 - p : p;
-        const int nl = s == S - 1 ? nl_last : 64;
+        const int nl = s == S - 1 ? nl_last : kStripCols;
         const i64 base = pad + (i64)s * full_strip;
         const bool has_in = p > 0, has_out = p < S - 1;
         // stream j runs between the strips at positions j and j+1 of the walk
         const double* bi = bnd + (i64)(p > 0 ? p - 1 : 0) * bstride;
         double* bo = bnd + (i64)p * bstride;
-        const int in_shift = dir ? (s + 1 == S - 1 ? nl_last : 64) - 1 : 63;
-        const bool seed = dir ? (s == S - 1 && lane == nl - 1) : (s == 0 && lane == 0);
-        if (dir == 0) log_dispatch<false, false>(has_in, has_out, T, nl, seed, in_shift, 63, lp + base, out + base, bi, bo, none, none, status);
-        else log_dispatch<true, false>(has_in, has_out, T, nl, seed, in_shift, nl - 1, lp + base, out + base, bi, bo, none, none, status);
+        const int in_shift = dir ? (int)strip_lanes(s + 1 == S - 1 ? nl_last : kStripCols) - 1 : 63;
+        const int seed_col = dir ? (s == S - 1 ? nl - 1 : -1) : (s == 0 ? 0 : -1);
+        if (dir == 0) log_dispatch<false, false>(has_in, has_out, T, nl, seed_col, in_shift, 63, lp.l + base, out + base, bi, bo, none, none, status);
+        else log_dispatch<true, false>(has_in, has_out, T, nl, seed_col, in_shift, (int)strip_lanes(nl) - 1, lp.l + base, out + base, bi, bo, none, none, status);
         __threadfence_block();
     }
 }
@@ -752,13 +920,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void k_lattice(
 // Polls a wait inside k_lattice may spend; settable from the host so that the give-up path can be
 // exercised (with a limit of 1 a strip that has to wait for its feeder gives up at once, and every
 // wave still leaves the kernel normally).
-static int g_wait_limit = kSpinLimit;
-void set_wait_limit(int polls) { g_wait_limit = polls > 0 ? polls : kSpinLimit; }
-static int wait_limit() { return g_wait_limit; }
+static std::atomic<int> g_wait_limit{kSpinLimit};
+void set_wait_limit(int polls) { g_wait_limit.store(polls > 0 ? polls : kSpinLimit, std::memory_order_relaxed); }
+static int wait_limit() { return g_wait_limit.load(std::memory_order_relaxed); }
 
 // one wave per strip of the longest label sequence the call admits, up to the concurrent limit
 static int lattice_waves(const Batch& b) {
-    const i64 strips = (b.max_u + 64) / 64;
+    const i64 strips = strip_count(b.max_u + 1);
     return (int)(strips < kMaxWaves ? (strips < 1 ? 1 : strips) : kMaxWaves);
 }
 
@@ -781,29 +949,22 @@ __device__ __forceinline__ bool linear_alpha(int mode, int S) { return (mode & 3
 __device__ __forceinline__ bool linear_beta(int mode, int S) { return (mode & 5) == 0 && S <= kMaxWaves; }
 
 // Base-2 logarithm of the lattice value stored for cell (t,u): either stored as such (log walk),
-// or as value * 2^C with C recorded per block of kPF steps of the strip's walk (linear walk).
+// or as value * 2^C with C recorded per lane and block of kPF steps of the strip's walk (linear walk).
 struct LatticeView {
     const double* v;
     const int* scale;
     i64 pad;
     int T, Up;
     bool linear, beta;
-    // value at `slot`, column l of the nl-wide strip that starts at slot `base`, written at step k
-    // of its walk
-    __device__ __forceinline__ double at_slot(i64 slot, i64 base, int k, int nl, int l) const {
-        const double x = v[slot];
-        if (!linear) return x;
-        const int C = scale[(base >> 4) + (k / kPF) * nl + l];
-        const int ex = __builtin_amdgcn_frexp_exp(x);
-        const float mant = (float)__builtin_amdgcn_frexp_mant(x);
-        return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
+    // where the scale of the value that lane l of the `lanes`-lane strip starting at slot `base`
+    // wrote at step k of its walk is kept
+    __device__ __forceinline__ i64 scale_index(i64 base, int k, int lanes, int l) const {
+        return (base >> 4) + (i64)(k / kPF) * lanes + l;
     }
-    // the same in two steps, so that a caller can have many loads in flight before it converts
-    __device__ __forceinline__ i64 scale_index(i64 base, int k, int nl, int l) const {
-        return (base >> 4) + (k / kPF) * nl + l;
-    }
+    // in two steps (load, convert), so that a caller can have many loads in flight before it converts
     __device__ __forceinline__ double convert(double x, int C) const {
         if (!linear) return x;
+        // log2 x = exponent + log2(mantissa), mantissa in [0.5, 1)
         const int ex = __builtin_amdgcn_frexp_exp(x);
         const float mant = (float)__builtin_amdgcn_frexp_mant(x);
         return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
@@ -812,16 +973,13 @@ struct LatticeView {
         const i64 slot = pad + lattice_slot(t, u, T, Up);
         const double x = v[slot];
         if (!linear) return x;
-        const int s = u >> 6, l = u & 63;
-        const int nl = Up - (s << 6) < 64 ? Up - (s << 6) : 64;
+        const int s = u >> kStripShift, l = (u & (kStripCols - 1)) >> 1;
+        const int nl = Up - (s << kStripShift) < kStripCols ? Up - (s << kStripShift) : kStripCols;
+        const int lanes = (int)strip_lanes(nl);
         const int q = t + l;
-        const int k = beta ? (T + nl - 2 - q) : q;
-        const i64 base = pad + (i64)s * strip_rows(T, 64) * 64;
-        const int C = scale[(base >> 4) + (k / kPF) * nl + l];
-        // log2 x = exponent + log2(mantissa), mantissa in [0.5, 1)
-        const int ex = __builtin_amdgcn_frexp_exp(x);
-        const float mant = (float)__builtin_amdgcn_frexp_mant(x);
-        return x == 0.0 ? -INFINITY : (double)(ex - C) + (double)fast_log2(mant);
+        const int k = beta ? (T + lanes - 2 - q) : q;
+        const i64 base = pad + (i64)s * strip_rows(T, kStripCols) * kStripCols;
+        return convert(x, scale[scale_index(base, k, lanes, l)]);
     }
 };
 
@@ -849,20 +1007,24 @@ __device__ __forceinline__ void finish_costs(bool wrote, int N, float* costs, fl
     }
 }
 
-// One wave per chunk: kFillRows consecutive rows of one strip of one sequence.  Which sequence,
-// strip and rows is the same for the whole wave, so the search through the chunk offsets and all
-// the index arithmetic run once per wave on the scalar unit; a lane keeps one column (64 / nl rows
-// share a pass when the strip is narrow), reads alpha, beta and the cell records of its slots at
-// consecutive addresses (the strip layout is diagonal to the row order) and scatters the 8-byte
-// results to the row order.  The two successors of cell (t,u) sit one strip row further: same column
-// (t+1,u) and next column (t,u+1); only the last column of a strip looks into the next strip.
-// The grid is fixed; waves stride over the chunks, whose number only the device knows.
+// One wave per chunk: kFillSlots consecutive slots of the cell rows of one strip of one sequence.
+// Which sequence and strip is the same for the whole wave, so the search through the chunk offsets
+// and the strip's geometry run once per wave on the scalar unit; a lane takes every 64th slot of the
+// chunk, reads alpha, beta and the cell records at consecutive addresses (the strip layout is
+// diagonal to the row order) and scatters the 8-byte results to the row order.  The successors of
+// cell (t,u) sit close by: (t+1,u) one strip row further in the same column; (t,u+1) in the next
+// slot for a lane's first column, one strip row further for its second; only the last column of a
+// strip looks into the next strip.  The grid is fixed; waves stride over the chunks, whose number
+// only the device knows.  A poisoned sequence (bad label, lattice wait that ran out) gets zero
+// gradients next to its NaN cost.
+constexpr int kFillPasses = kFillSlots / 64;
+
 __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const int* __restrict__ ly,
                                                const i64* __restrict__ row_off,
                                                const i64* __restrict__ pad_off,
                                                const i64* __restrict__ fill_off,
                                                const int* __restrict__ seqmode, int N, i64 R,
-                                               const LpCell* __restrict__ lp,
+                                               const float2* __restrict__ lpl,
                                                const double* __restrict__ alpha, const double* __restrict__ beta,
                                                const int* __restrict__ scale_a, const int* __restrict__ scale_b,
                                                float2* __restrict__ grads, float* costs, float* reduced,
@@ -908,71 +1070,86 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
         bool wrote = false;
         if (pad >= 0) {
             const int Up = U + 1;
-            const int S = (Up + 63) >> 6;
-            const unsigned per_full = (unsigned)strip_chunks(T, 64);
+            const int S = (int)strip_count(Up);
+            const unsigned per_full = (unsigned)strip_chunks(T, kStripCols);
             const unsigned local = (unsigned)(c - f0);
             unsigned s = local / per_full;
             s = s < (unsigned)(S - 1) ? s : (unsigned)(S - 1);
-            const int q0 = (int)(local - s * per_full) * kFillRows;  // first row of the chunk (0 = the strip's first cell row)
-            const int nl = (int)s == S - 1 ? Up - ((int)s << 6) : 64;
-            const int Q = T + nl - 1;
-            const i64 full = strip_rows(T, 64) * 64;
+            const int nl = (int)s == S - 1 ? Up - ((int)s << kStripShift) : kStripCols;
+            const int lanes = (int)strip_lanes(nl);
+            const int Q = T + lanes - 1;  // rows of the strip that hold cells
+            const i64 full = strip_rows(T, kStripCols) * kStripCols;
             const i64 base = pad + (i64)s * full;
+            // first slot of the chunk, counted from the strip's first cell row, as (row, column)
+            const unsigned i0 = (local - s * per_full) * (unsigned)kFillSlots;
+            const unsigned q_first = i0 / (unsigned)nl;
+            const int c_first = (int)(i0 - q_first * (unsigned)nl);
+            const float inv_nl = 1.0f / (float)nl;
             // the strip after this one, for the cells of this strip's last column
-            const int nl2 = (int)s + 1 < S ? ((int)s + 2 == S ? Up - (((int)s + 1) << 6) : 64) : 1;
+            const int nl2 = (int)s + 1 < S ? ((int)s + 2 == S ? Up - (((int)s + 1) << kStripShift) : kStripCols) : 1;
+            const int lanes2 = (int)strip_lanes(nl2);
             const i64 base2 = base + full;
             LatticeView A, Bv;
             A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
             Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
             const double b00 = Bv.log2_at(0, 0);  // all values are base-2 logarithms
-            const int rpp = 64 / nl;  // rows per pass
-            const int rr = lane / nl, l = lane - rr * nl;
-            const int u = ((int)s << 6) + l;
             // every pass's loads go out before any of them is used: lanes without a cell read
-            // the strip's first cell row instead and drop the result
-            struct Raw { double a, bd, bn; LpCell cell; int ca, cbd, cbn; int t; bool ok; };
-            Raw raw[kFillRows];
+            // the strip's first cell instead and drop the result
+            struct Raw { double a, bd, bn; float2 cell; int ca, cbd, cbn; int t, u; bool ok; };
+            Raw raw[kFillPasses];
 #pragma unroll
-            for (int pass = 0; pass < kFillRows; ++pass) {
+            for (int pass = 0; pass < kFillPasses; ++pass) {
                 Raw& w = raw[pass];
-                const int p0 = pass * rpp;
-                const int q = q0 + p0 + rr;
+                // slot c_first + 64*pass + lane of the rows from q_first on; at most
+                // nl + kFillSlots < 2^9, so the quotient by nl is exact in fp32
+                const int il = c_first + pass * 64 + lane;
+                const int dqr = (int)(((float)il + 0.5f) * inv_nl);
+                const int q = (int)q_first + dqr;
+                const int col = il - dqr * nl;
+                const int l = col >> 1;
                 const int t = q - l;
-                w.ok = rr < rpp && p0 + rr < kFillRows && q < Q && t >= 0 && t < T;
-                const int qs = w.ok ? q : 0, ls = w.ok ? l : 0;
+                w.ok = q < Q && t >= 0 && t < T;
+                const int qs = w.ok ? q : 0, cs = w.ok ? col : 0, ls = w.ok ? l : 0;
                 w.t = qs - ls;
-                const i64 slot = base + (i64)(qs + kRowShift) * nl + ls;
-                const int kb = max(T + nl - 2 - (qs + 1), 0);  // step of the beta walk that wrote strip row qs + 1
-                const bool inside = ls + 1 < nl || !w.ok || (int)s + 1 >= S;  // else: column 0 of the next strip, row t
-                const i64 slot_n = inside ? slot + nl + 1 : base2 + (i64)(w.t + kRowShift) * nl2;
+                w.u = ((int)s << kStripShift) + cs;
+                const i64 slot = base + (i64)(qs + kRowShift) * nl + cs;
+                // (t+1,u): same column, next strip row, written at step Q-2-q of the beta walk.
+                // (t,u+1): the lane's second column in the same row (step Q-1-q), or the next lane's
+                // first column one row further (step Q-2-q), or column 0 of the next strip in row t.
+                const bool second = (cs & 1) != 0;
+                const bool inside = cs + 1 < nl || !w.ok || (int)s + 1 >= S;
+                const i64 slot_n = inside ? (second ? slot + nl + 1 : slot + 1) : base2 + (i64)(w.t + kRowShift) * nl2;
+                const int kb_d = max(Q - 2 - qs, 0);
                 w.a = alpha[slot];
-                w.cell = lp[slot];
+                w.cell = lpl[slot];
                 w.bd = beta[slot + nl];
                 w.bn = beta[slot_n];
                 w.ca = w.cbd = w.cbn = 0;
-                if (A.linear) w.ca = scale_a[A.scale_index(base, qs, nl, ls)];
+                if (A.linear) w.ca = scale_a[A.scale_index(base, qs, lanes, ls)];
                 if (Bv.linear) {
-                    w.cbd = scale_b[Bv.scale_index(base, kb, nl, ls)];
-                    w.cbn = scale_b[inside ? Bv.scale_index(base, kb, nl, min(ls + 1, nl - 1))
-                                           : Bv.scale_index(base2, max(T + nl2 - 2 - w.t, 0), nl2, 0)];
+                    w.cbd = scale_b[Bv.scale_index(base, kb_d, lanes, ls)];
+                    w.cbn = scale_b[inside ? (second ? Bv.scale_index(base, kb_d, lanes, min(ls + 1, lanes - 1))
+                                                     : Bv.scale_index(base, Q - 1 - qs, lanes, ls))
+                                           : Bv.scale_index(base2, max(T + lanes2 - 2 - w.t, 0), lanes2, 0)];
                 }
             }
+            const bool poisoned = (mode & kSeqPoisoned) != 0;
 #pragma unroll
-            for (int pass = 0; pass < kFillRows; ++pass) {
+            for (int pass = 0; pass < kFillPasses; ++pass) {
                 const Raw& w = raw[pass];
-                const int t = w.t;
+                const int t = w.t, u = w.u;
                 const i64 r = roff + (i64)t * Up + u;
                 if (!w.ok || r >= R) continue;
                 const double a = A.convert(w.a, w.ca);
                 float gb = 0.f, gl = 0.f;
-                if (t < T - 1) gb = -fast_exp2((float)(a + Bv.convert(w.bd, w.cbd) + (double)w.cell.l_blank - b00));
-                else if (u == U) gb = -fast_exp2((float)(a + (double)w.cell.l_blank - b00));
-                if (u < U) gl = -fast_exp2((float)(a + Bv.convert(w.bn, w.cbn) + (double)w.cell.l_label - b00));
-                grads[r] = make_float2(gb, gl);
+                if (t < T - 1) gb = -fast_exp2((float)(a + Bv.convert(w.bd, w.cbd) + (double)w.cell.x - b00));
+                else if (u == U) gb = -fast_exp2((float)(a + (double)w.cell.x - b00));
+                if (u < U) gl = -fast_exp2((float)(a + Bv.convert(w.bn, w.cbn) + (double)w.cell.y - b00));
+                grads[r] = poisoned ? make_float2(0.f, 0.f) : make_float2(gb, gl);
                 if (t == T - 1 && u == U) {
                     float cost;
-                    if (cost_rule(a + (double)w.cell.l_blank, b00, &cost)) raise_flag(status, CWR_FLAG_FB_MISMATCH);
-                    costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : cost;
+                    if (cost_rule(a + (double)w.cell.x, b00, &cost)) raise_flag(status, CWR_FLAG_FB_MISMATCH);
+                    costs[n] = poisoned ? __int_as_float(0x7fc00000) : cost;
                     wrote = true;
                 }
             }
@@ -981,16 +1158,17 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
     }
 }
 
-// Waves k_fill is launched with: one GPU full of them (8 per SIMD), never more than the chunks a batch of R rows in N sequences can have (a chunk holds at least one
-// row of cells of the lattice, and every strip ends with one partly filled chunk).
+// Waves k_fill is launched with: one GPU full of them (8 per SIMD), never more than the chunks a
+// batch of R rows in N sequences can have (a strip's cell rows hold its cells and, per lane, one
+// row of padding; every strip ends with one partly filled chunk).
 int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* grads, float* costs,
                 float* reduced) {
     if (b.R == 0) return CWR_OK;
-    const i64 strips = (b.max_u + 64) / 64;
-    i64 waves = b.R / kFillRows + (i64)b.N * strips * 6 + 1;
+    const i64 strips = strip_count(b.max_u + 1);
+    i64 waves = b.R / kFillSlots + (i64)b.N * strips * (64 * kStripCols / kFillSlots + 1) + 1;
     if (waves > 8192) waves = 8192;
     CWR_LAUNCH(k_fill, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
-                       ws.pad_off, ws.fill_off, ws.seqmode, b.N, b.R, ws.lp, ws.alpha, ws.beta, ws.scale_a,
+                       ws.pad_off, ws.fill_off, ws.seqmode, b.N, b.R, ws.lp.l, ws.alpha, ws.beta, ws.scale_a,
                        ws.scale_b, reinterpret_cast<float2*>(grads), costs, reduced, b.status);
     (void)rowinfo;  // rows of skipped sequences were given their zero record by the gather pass
     return check_launch();
@@ -1009,7 +1187,7 @@ __global__ __launch_bounds__(64) void k_cost_from_beta(const int* __restrict__ l
         LatticeView Bv;
         Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = lx[n]; Bv.Up = ly[n] + 1; Bv.beta = true;
         const int mode = seqmode[n];
-        Bv.linear = linear_beta(mode, (Bv.Up + 63) >> 6);
+        Bv.linear = linear_beta(mode, (int)strip_count(Bv.Up));
         costs[n] = (mode & kSeqPoisoned) ? __int_as_float(0x7fc00000) : (float)(-Bv.log2_at(0, 0) * (double)kLn2);
         wrote = true;
     }
@@ -1046,7 +1224,7 @@ __global__ __launch_bounds__(256) void k_export(const int* __restrict__ lx, cons
     double a = 0.0, b = 0.0;
     if (pad >= 0 && t < T && u < Up) {
         LatticeView A, Bv;
-        const int mode = seqmode[n], S = (Up + 63) >> 6;
+        const int mode = seqmode[n], S = (int)strip_count(Up);
         A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
         Bv.v = beta; Bv.scale = scale_b; Bv.pad = pad; Bv.T = T; Bv.Up = Up; Bv.linear = linear_beta(mode, S); Bv.beta = true;
         if (alphas_out) a = A.log2_at(t, u) * 0.6931471805599453;

@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_row(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    LpStore lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     // beyond 32 values per lane the register vector would be indexed through scratch memory:
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_rows(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    LpStore lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int RP = 64 / LPR;   // rows per pass
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_long(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    LpStore lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int VEC = Elem<T>::VEC;
     constexpr int KC = 4;
@@ -559,7 +559,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_small(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    LpStore lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     constexpr int RP = 64 / LPR;
     const int lane = threadIdx.x & 63;
@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void k_gather_fused_generic(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
+    LpStore lp, float* __restrict__ lse_out, int2* __restrict__ rowinfo,
     float2* __restrict__ grads_skipped, int* __restrict__ seqmode, int* __restrict__ status) {
     const int lane = threadIdx.x & 63;
     const i64 r = wave_first_row(1);
@@ -645,7 +645,7 @@ __global__ __launch_bounds__(256) void k_gather_logprob(
     const T* __restrict__ x, i64 R, int V, const int* __restrict__ lx, const int* __restrict__ ly,
     const int* __restrict__ y, i64 y_stride, i64 y_len, const i64* __restrict__ row_off,
     const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N, int blank,
-    LpCell* __restrict__ lp, int2* __restrict__ rowinfo, float2* __restrict__ grads_skipped,
+    LpStore lp, int2* __restrict__ rowinfo, float2* __restrict__ grads_skipped,
     int* __restrict__ seqmode, int* __restrict__ status) {
     const i64 r = (i64)blockIdx.x * 256 + threadIdx.x;
     if (r >= R) return;

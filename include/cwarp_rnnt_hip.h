@@ -80,27 +80,28 @@ int cwr_version(void);
 const char* cwr_strerror(int status);
 
 /* Bytes of scratch cwr_forward / cwr_loss need for a batch of N sequences, R rows and at most
- * max_u labels per sequence.  The scratch holds the gathered cell records, alpha and beta
+ * max_u labels per sequence.  The scratch holds the gathered blank / label records, alpha and beta
  * (O(R) plus a per-sequence padding that grows with max_u, so pass a tight max_u); nothing in it
  * is needed by cwr_backward.  Must be 256-byte aligned. */
 size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
 
 /* Location of the lattice state inside the workspace after cwr_forward, for analysis tools (the
  * reference returns alpha and beta, cwarp_cuda_rnnt_kernel.cu:383-384).  which:
- *   0  gathered cell records, 16 bytes per cell: fp32 P(blank), P(label), log2 P(blank),
- *      log2 P(label)
+ *   0  gathered probabilities, 8 bytes per cell: fp32 P(blank), P(label)
+ *   7  gathered log-probabilities, 8 bytes per cell: fp32 log2 P(blank), log2 P(label)
  *   1  alpha, 2  beta: one fp64 per cell
  *   3  pad_off: N+1 int64, first cell slot of each sequence, -1 for a skipped sequence
  *   4  seqmode: N+1 int32 (N used), how the sequence was walked.  0 = both directions in the
  *      scaled linear domain; bit 0 = both in the log domain (log-probs outside what the linear
  *      walk carries); bit 1 / bit 2 = alpha / beta was walked again in the log domain.  A sequence
- *      with more than 8 strips of 64 labels is always in the log domain.
+ *      with more than 8 strips of 128 labels is always in the log domain.
  *   5  scale_a, 6  scale_b: int32 scale exponents of the linear-domain walk
  * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U).
  * Log-domain values are base-2 logarithms (multiply by ln 2).  Linear-domain values are
- * value * 2^C: for strip s = u/64 of width nl = min(64, U+1-64s), column l = u%64, the walk step is
- * k = t+l (alpha) or T+nl-2-(t+l) (beta) and
- * C = scale[(pad_off[n] + s*(T+127)*64)/16 + (k/16)*nl + l].  cwr_export_lattice does this. */
+ * value * 2^C: a strip s = u/128 of width nl = min(128, U+1-128s) is walked by L = ceil(nl/2) lanes,
+ * lane l = (u%128)/2 holding columns 2l and 2l+1; the walk step is k = t+l (alpha) or
+ * T+L-2-(t+l) (beta) and C = scale[(pad_off[n] + s*(T+127)*128)/16 + (k/16)*L + l].
+ * cwr_export_lattice does this. */
 int cwr_workspace_section(int64_t N, int64_t R, int64_t max_u, int which, size_t* offset, size_t* bytes);
 int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U); /* host helper */
 

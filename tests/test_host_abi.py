@@ -55,27 +55,31 @@ def test_workspace_size_is_monotone_and_bounded():
     huge = lib.cwr_workspace_bytes(32, 1000, 10 ** 9)
     assert huge < 1000 * 128 * 33 + 10 ** 6
     off, nbytes = C.c_size_t(), C.c_size_t()
-    for which in range(7):
+    for which in range(8):
         assert lib.cwr_workspace_section(32, 300000, 80, which, C.byref(off), C.byref(nbytes)) == 0
         assert off.value + nbytes.value <= base and off.value % 256 == 0
     assert lib.cwr_workspace_section(32, 300000, 80, 9, C.byref(off), C.byref(nbytes)) == 4
 
 
 def test_lattice_slot_is_a_bijection_into_the_bound():
-    """Every cell of a T x (U+1) lattice gets its own slot below lattice size, for shapes around
-    the 64-column strip width."""
+    """Every cell of a T x (U+1) lattice gets its own slot below the lattice size, for shapes around
+    the 128-column strip width (two columns per lane: even and odd widths), and the two cells of a
+    lane lie next to each other in one strip row."""
     lib = _lib.load()
-    for T, U in [(1, 0), (1, 70), (5, 3), (3, 63), (3, 64), (2, 130), (40, 65)]:
+    for T, U in [(1, 0), (1, 70), (5, 3), (3, 126), (3, 127), (3, 128), (2, 260), (40, 129), (7, 4)]:
         slots = set()
         for t in range(T):
             for u in range(U + 1):
                 s = lib.cwr_lattice_slot(t, u, T, U)
                 assert s >= 0
                 slots.add(s)
+                if u % 2 == 1:
+                    assert s == lib.cwr_lattice_slot(t, u - 1, T, U) + 1
         assert len(slots) == T * (U + 1)
-        strips = U // 64 + 1
-        nl = U + 1 - 64 * (strips - 1)
-        size = (strips - 1) * (T + 63 + 64) * 64 + (T + nl - 1 + 64) * nl
+        strips = U // 128 + 1
+        nl = U + 1 - 128 * (strips - 1)
+        lanes = (nl + 1) // 2
+        size = (strips - 1) * (T + 63 + 64) * 128 + (T + lanes - 1 + 64) * nl
         assert max(slots) < size
         assert lib.cwr_lattice_slot(T, 0, T, U) == -1 and lib.cwr_lattice_slot(0, U + 1, T, U) == -1
 
@@ -290,3 +294,17 @@ def test_joint_entry_points_reject_invalid_calls_on_the_host():
                                      A, None)
 
     assert fwd(dtype=_lib.F32) == 2 and fwd(H=40) == 4 and fwd(h=None) == 1 and fwd(w=A + 2) == 6
+
+
+def test_build_step_flags_a_scalar_select_on_a_stale_condition_code():
+    """The build refuses device assembly in which a scalar select reads a condition code that only an
+    unrelated instruction set (seen from hipcc for a select on a loop counter kept in a vector
+    register); a select behind its own scalar compare passes."""
+    from compactwarprnntloss_amd.build import stale_scc_reads
+    bad = "\n".join(["\ts_add_i32 s12, s12, s52", "\tv_add_u32_e32 v67, 1, v67", "\tv_cmp_eq_u32_e32 vcc, s20, v67",
+                     "\ts_cselect_b32 s3, 0x7fffffff, s15", "\tds_write_b32 v91, v95"])
+    good = "\n".join(["\ts_add_i32 s58, s58, 1", "\tv_cmp_eq_u32_e32 vcc, s20, v67", "\ts_cmp_lg_u32 s58, s74",
+                      "\ts_cselect_b32 s3, s2, 0x7fffffff"])
+    via_mask = "\n".join(["\tv_cmp_eq_u32_e32 vcc, s20, v67", "\ts_and_b64 vcc, vcc, exec", "\ts_cselect_b32 s12, 0x7fffffff, s3"])
+    assert [n for n, _ in stale_scc_reads(bad)] == [4]
+    assert stale_scc_reads(good) == [] and stale_scc_reads(via_mask) == []
