@@ -11,8 +11,9 @@ one synthetic batch that is already resident in HBM.  Prints ONE JSON line.
              them again in the backward pass, write the gradient (R = sum T_i*(U_i+1)).
   roofline   the gradient kernel (the dominant one: 2/3 of the bytes) timed on its own with
              HIP events on the stream it is launched on, against the 8 TB/s HBM peak.
-  cpu_baseline  the float64 NumPy oracle timed on this host on a bounded sample of the same
-             batch; its outputs double as the parity check of the run.
+  cpu_baseline  the C restatement of the float64 oracle (OpenMP, all host cores of the process)
+             timed on whole passes over the same batch for a bounded time; its outputs double as
+             the parity check of the run.
 """
 from __future__ import annotations
 
@@ -52,37 +53,39 @@ def measured_traffic(kernel: str, config: int):
 
 
 def cpu_baseline(cfg, x_cpu, budget_s, dev_out):
-    """Time the NumPy oracle on the sequences of the batch, one after the other, for about half the
-    budget at least (going round the batch again if it is done sooner) and never beyond the budget;
-    the first time round, compare the device results on those sequences."""
+    """Time the C restatement of the oracle (oracle/rnnt_oracle_c.c: float64 arithmetic, OpenMP over
+    the sequences of the batch, every host core the process may use) on whole passes over the same
+    batch, for about the budget; the first pass's outputs double as the parity check of the device
+    results (the C restatement is itself pinned to the NumPy oracle in tests/test_oracle_pins.py)."""
     import torch
-    from oracle import rnnt_oracle as orc
-    off = orc.row_offsets_i64(cfg["lx"], cfg["ly"])
+    from oracle import build_c
+    lib = build_c.load()
+    x32 = x_cpu.to(dtype=torch.float32).numpy()
+    N, V = cfg["N"], cfg["V"]
     esize = x_cpu.element_size()
-    t_used, n_done, bytes_done = 0.0, 0, 0
-    loss_rel, grad_abs = 0.0, 0.0
-    N = cfg["N"]
+    go = np.full(N, 1.0 / N)
+    t_used, passes = 0.0, 0
+    loss_rel = grad_abs = 0.0
     while True:
-        n = n_done % N
-        xs = x_cpu[off[n]:off[n + 1]].to(dtype=torch.float64).numpy()
-        lab = cfg["y_padded"][n:n + 1]
         t0 = time.perf_counter()
-        ref = orc.loss_and_grad(xs, cfg["lx"][n:n + 1], lab, cfg["ly"][n:n + 1], 0, "fused",
-                                grad_out=np.array([1.0 / N]))
+        ref = build_c.loss_and_grad(lib, x32, cfg["lx"], cfg["y_padded"], cfg["ly"], 0, True, go, want_G=False)
         dt = time.perf_counter() - t0
         t_used += dt
-        n_done += 1
-        bytes_done += xs.shape[0] * cfg["V"] * 3 * esize
-        if n_done <= N:
-            loss_rel = max(loss_rel, abs(dev_out["costs"][n] - ref["costs"][0]) / abs(ref["costs"][0]))
-            grad_abs = max(grad_abs, float(np.abs(dev_out["grad"](off[n], off[n + 1]) - ref["grad"]).max()))
-        if t_used + dt > budget_s or (n_done >= N and n_done % N == 0 and t_used >= 0.5 * budget_s):
+        passes += 1
+        if passes == 1:
+            loss_rel = float(np.max(np.abs(dev_out["costs"] - ref["costs"]) / np.abs(ref["costs"])))
+            step = 1 << 16
+            for a in range(0, x32.shape[0], step):
+                grad_abs = max(grad_abs, float(np.abs(dev_out["grad"](a, a + step) - ref["grad"][a:a + step]).max()))
+        del ref
+        if t_used + dt > budget_s:
             break
-    checked = min(n_done, N)
-    return dict(value=bytes_done / t_used / 1e9, unit="GB/s", cores=1, kind="port",
-                sample=f"float64 NumPy oracle, {n_done} sequence passes over the {N} sequences of the same "
-                       f"batch ({n_done / N:.1f} batches), {t_used:.1f} s",
-                ), dict(loss_rel_err=loss_rel, grad_abs_err=grad_abs, sequences_checked=checked)
+    bytes_done = passes * x32.shape[0] * V * 3 * esize
+    cores = int(lib.rnnt_oracle_c_threads())
+    return dict(value=bytes_done / t_used / 1e9, unit="GB/s", cores=cores, kind="port",
+                sample=f"C restatement of the float64 oracle (OpenMP over sequences, {cores} threads of "
+                       f"{os.cpu_count()} host cpus), {passes} whole passes over the same batch, {t_used:.1f} s",
+                ), dict(loss_rel_err=loss_rel, grad_abs_err=grad_abs, sequences_checked=N)
 
 
 def main():
@@ -197,6 +200,26 @@ def main():
     fwd_ms = timed(lambda: pkg.rnnt_forward(xd, lx, y, ly, 0, True))
     nograd_ms = timed(lambda: pkg.rnnt_forward(xd, lx, y, ly, 0, True, with_grad=False))
 
+    # Latency breakdown of the forward call: HIP events between its four stages (a measurement hook of
+    # the library; each figure holds the kernel and the dependency gap in front of it), the gradient
+    # pass from the backward call above.  One anti-diagonal = one frame or label of the sequence with
+    # the most of them; the lattice walk is a serial chain over those.
+    import ctypes as C
+    lib = pkg._lib.load()
+    stage = (C.c_float * 4)()
+    lat_runs = []
+    for _ in range(max(10, args.steps // 2)):
+        rc = lib.cwr_debug_forward_stage_times(
+            xd.data_ptr(), pkg.loss._DTYPES[xd.dtype], R, V, lx.data_ptr(), ly.data_ptr(), y.data_ptr(), y.size(1),
+            y.numel(), N, 0, pkg._lib.MODE_FUSED, st.max_u, st.workspace.data_ptr(), st.workspace.numel(),
+            st.row_off.data_ptr(), st.lab_off.data_ptr(), st.status.data_ptr(), st.rowinfo.data_ptr(),
+            st.lse.data_ptr(), st.grads.data_ptr(), costs.data_ptr(), torch.cuda.current_stream().cuda_stream, stage)
+        if rc != 0:
+            sys.exit("cwr_debug_forward_stage_times: " + pkg._lib.strerror(rc))
+        lat_runs.append(list(stage))
+    lat = [sorted(r[i] for r in lat_runs)[len(lat_runs) // 2] for i in range(4)]  # medians
+    diagonals = int((cfg["lx"].astype(np.int64) + cfg["ly"]).max())
+
     grad_bytes = R * V * 2 * esize
     achieved = grad_bytes / (bwd_ms * 1e-3) / 1e9
     traffic, traffic_source = measured_traffic("k_grad", args.config)
@@ -220,6 +243,12 @@ def main():
                     "max": round(per_step[-1], 4)},
         "breakdown_ms": {"forward_call": round(fwd_ms, 4), "backward_call": round(bwd_ms, 4),
                          "forward_nograd_call": round(nograd_ms, 4)},
+        "latency_us": {"offsets": round(lat[0], 2), "gather": round(lat[1], 2), "lattice": round(lat[2], 2),
+                       "fill": round(lat[3], 2), "grad": round(bwd_ms * 1e3, 2),
+                       "lattice_ns_per_diagonal": round(lat[2] * 1e3 / diagonals, 1),
+                       "diagonals_longest_sequence": diagonals,
+                       "how": "medians of HIP-event intervals between the stages of one forward call "
+                              "(cwr_debug_forward_stage_times); grad = the backward call"},
         "roofline": {"bound": "hbm", "kernel": "k_grad (cwr_backward)", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic, "traffic_source": traffic_source},

@@ -40,6 +40,9 @@ SIGNATURES = {
     "cwr_offsets": (C.c_int, [_p, _p, _i64, _i64, _p, _p, _p, _p]),
     "cwr_forward": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                               _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "cwr_debug_forward_stage_times": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int,
+                                                _i64, _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p,
+                                                C.POINTER(C.c_float)]),
     "cwr_forward_noalloc": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,
                                       _p, _p, _p, _p, _p, _p, _p, _p]),
     "cwr_loss": (C.c_int, [_p, C.c_int, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, C.c_int, _i64,

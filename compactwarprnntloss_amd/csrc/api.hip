@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <mutex>
 
+#include "../../include/cwarp_rnnt_hip_testing.h"
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
@@ -229,41 +230,60 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R, int6
                           static_cast<hipStream_t>(stream));
 }
 
+// Everything the host can judge about a forward call's arguments, before any HIP call.
+static int check_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
+                         const int32_t* y, int64_t y_len, int64_t N, int32_t blank, int mode, int64_t max_u,
+                         const int64_t* row_off, const int64_t* lab_off, const int32_t* status,
+                         const int32_t* rowinfo, const float* lse, const float* grads, const float* costs,
+                         const float* reduced, bool with_grad, bool joint) {
+    int rc = check_common(x, !joint, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+    if (rc != CWR_OK) return rc;
+    if (max_u < 0) return CWR_ERR_SHAPE;
+    if (!row_off || !lab_off || !status) return CWR_ERR_NULL;
+    if (N > 0 && !costs) return CWR_ERR_NULL;
+    if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
+    if (R > 0 && (!rowinfo || (with_grad && !grads))) return CWR_ERR_NULL;
+    if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
+        misaligned(rowinfo, 8) || misaligned(grads, 8) || misaligned(costs, 4) || misaligned(reduced, 4))
+        return CWR_ERR_ALIGN;
+    return CWR_OK;
+}
+
 static int forward_impl(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, void* workspace, size_t workspace_bytes_, int64_t* row_off,
                         int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse, float* grads,
                         float* costs, float* reduced, void* stream, bool with_grad,
-                        const JointOperands* joint = nullptr) {
-    int rc = check_common(x, joint == nullptr, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+                        const JointOperands* joint = nullptr, hipEvent_t* marks = nullptr) {
+    int rc = check_forward(x, dtype, R, V, lx, ly, y, y_len, N, blank, mode, max_u, row_off, lab_off, status,
+                           rowinfo, lse, grads, costs, reduced, with_grad, joint != nullptr);
     if (rc != CWR_OK) return rc;
-    if (max_u < 0) return CWR_ERR_SHAPE;
-    if (!row_off || !lab_off || !status) return CWR_ERR_NULL;
-    if (N > 0 && !costs) return CWR_ERR_NULL;
     if (!workspace) return CWR_ERR_NULL;
-    if (R > 0 && mode == CWR_MODE_FUSED && !lse) return CWR_ERR_NULL;
-    if (R > 0 && (!rowinfo || (with_grad && !grads))) return CWR_ERR_NULL;
-    if (misaligned(row_off, 8) || misaligned(lab_off, 8) || misaligned(status, 4) || misaligned(lse, 4) ||
-        misaligned(rowinfo, 8) ||
-        misaligned(grads, 8) || misaligned(costs, 4) || misaligned(reduced, 4) || misaligned(workspace, 256))
-        return CWR_ERR_ALIGN;
+    if (misaligned(workspace, 256)) return CWR_ERR_ALIGN;
     Workspace ws;
     if (!carve_workspace(workspace, workspace_bytes_, N, R, max_u, &ws)) return CWR_ERR_SHAPE;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // marks (measurement hook only): five events, recorded in front of and behind the four stages
+    auto mark = [&](int i) { if (marks) (void)hipEventRecord(marks[i], s); };
+    mark(0);
     rc = launch_offsets(lx, ly, N, R, max_u, ws.slot_cap, ws.bnd_cap, reinterpret_cast<i64*>(row_off),
                         reinterpret_cast<i64*>(lab_off), ws.pad_off, ws.fill_off, ws.bnd_off, ws.seqmode, status, costs,
                         reduced, s);
     if (rc != CWR_OK) return rc;
+    mark(1);
     Batch b = make_batch(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, row_off, lab_off,
                          status, stream);
     rc = joint ? launch_joint_gather(b, ws, *joint, lse, rowinfo, with_grad ? grads : nullptr)
                : launch_gather(b, ws, lse, rowinfo, with_grad ? grads : nullptr);
     if (rc != CWR_OK) return rc;
+    mark(2);
     rc = launch_lattice(b, ws, !with_grad);
     if (rc != CWR_OK) return rc;
-    if (with_grad) return launch_fill(b, ws, rowinfo, grads, costs, reduced);
-    return launch_cost_from_beta(b, ws, costs, reduced);
+    mark(3);
+    rc = with_grad ? launch_fill(b, ws, rowinfo, grads, costs, reduced) : launch_cost_from_beta(b, ws, costs, reduced);
+    mark(4);
+    return rc;
 }
 
 int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
@@ -275,14 +295,45 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V, const int32_t* l
                         true);
 }
 
+int cwr_debug_forward_stage_times(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx,
+                                  const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N,
+                                  int32_t blank, int mode, int64_t max_u, void* workspace, size_t workspace_bytes_,
+                                  int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
+                                  float* grads, float* costs, void* stream, float* stage_us) {
+    if (!stage_us) return CWR_ERR_NULL;
+    hipEvent_t ev[5];
+    int made = 0;
+    int rc = CWR_OK;
+    for (; made < 5; ++made) {
+        const hipError_t e = hipEventCreate(&ev[made]);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; rc = CWR_ERR_RUNTIME; break; }
+    }
+    if (rc == CWR_OK)
+        rc = forward_impl(x, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, mode, max_u, workspace,
+                          workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream,
+                          true, nullptr, ev);
+    if (rc == CWR_OK) {
+        const hipError_t e = hipEventSynchronize(ev[4]);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; rc = CWR_ERR_RUNTIME; }
+    }
+    for (int i = 0; rc == CWR_OK && i < 4; ++i) {
+        float ms = 0.f;
+        const hipError_t e = hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; rc = CWR_ERR_RUNTIME; }
+        stage_us[i] = ms * 1000.f;
+    }
+    for (int i = 0; i < made; ++i) (void)hipEventDestroy(ev[i]);
+    return rc;
+}
+
 int cwr_forward_noalloc(const void* x, int dtype, int64_t R, int64_t V, const int32_t* lx, const int32_t* ly,
                         const int32_t* y, int64_t y_stride, int64_t y_len, int64_t N, int32_t blank, int mode,
                         int64_t max_u, int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo,
                         float* lse, float* grads, float* costs, void* stream) {
     // everything the host can judge first, so that a call that cannot run touches no GPU
-    int rc = check_common(x, true, dtype, R, V, lx, ly, y, y_len, N, blank, mode);
+    int rc = check_forward(x, dtype, R, V, lx, ly, y, y_len, N, blank, mode, max_u, row_off, lab_off, status,
+                           rowinfo, lse, grads, costs, nullptr, true, false);
     if (rc != CWR_OK) return rc;
-    if (max_u < 0) return CWR_ERR_SHAPE;
     const size_t need = workspace_bytes(N, R, max_u);
     if (need > (size_t)CWR_NOALLOC_SCRATCH_BYTES) return CWR_ERR_TOO_LARGE;
     void* ws = nullptr;
@@ -322,7 +373,7 @@ int cwr_joint_backward(const void* h, const void* w, const float* bias, int dtyp
     if (!h || !w || !rowinfo || !grads || !lse || !grad_costs || !dlogits) return CWR_ERR_NULL;
     if (misaligned(h, 16) || misaligned(w, 16) || misaligned(bias, 4) || misaligned(rowinfo, 8) ||
         misaligned(grads, 8) || misaligned(lse, 4) || misaligned(grad_costs, 4) ||
-        misaligned(dlogits, (V & 3) == 0 ? 8 : 2))  // runs of four entries leave as 8-byte stores
+        misaligned(dlogits, (V & 7) == 0 ? 16 : ((V & 3) == 0 ? 8 : 2)))  // rows leave as 16- / 8-byte stores
         return CWR_ERR_ALIGN;
     JointOperands j;
     j.h = h; j.w = w; j.bias = bias; j.H = H;

@@ -114,12 +114,6 @@ int64_t cwr_lattice_slot(int64_t t, int64_t u, int64_t T, int64_t U); /* host he
  * prints a warning.  Returns 0 otherwise, -1 for a NULL cost. */
 int cwr_cost_rule(double fwd_log2, double bwd_log2, float* cost);
 
-/* Diagnostic: the number of polls a wave of the lattice kernel spends waiting for the neighbouring
- * strip's wave before it gives up (CWR_FLAG_INTERNAL; the sequence's cost becomes NaN; every wave
- * still leaves the kernel normally).  polls <= 0 restores the default (about 4 million).  Process-
- * wide; meant for tests of that path. */
-void cwr_debug_wait_limit(int polls);
-
 /* Row and label offsets by a device prefix scan.
  *   row_off[n] = sum_{j<n} lx[j]*(ly[j]+1), n = 0..N   (N+1 entries, int64)
  *   lab_off[n] = sum_{j<n} ly[j],           n = 0..N   (N+1 entries, int64)
@@ -159,8 +153,12 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
  *   - cwr_workspace_bytes(N, R, max_u) must not exceed CWR_NOALLOC_SCRATCH_BYTES, else
  *     CWR_ERR_TOO_LARGE.  96 MiB: the N=32, T~175, U~50 batch (R = 3.1e5) needs 30 MiB, the
  *     long-form N=4, T~1250, U~300 batch (R = 1.5e6) 71 MiB.
+ *   - The array is part of the library's device code: every process that loads the library holds
+ *     96 MiB on every GPU it runs the library's kernels on, whether or not it ever calls this entry
+ *     point.
  *   - The first call on a GPU looks the array's address up (hipGetSymbolAddress); make it outside
- *     a stream capture.
+ *     a stream capture.  Calls with arguments the host can reject (null or misaligned pointers, bad
+ *     sizes) return before that look-up and touch no GPU.
  *   - Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams,
  *     two threads) race.  Calls in stream order on one stream are safe; nothing from an earlier
  *     call is relied on, the kernels initialise what they read.
@@ -305,6 +303,8 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
  * block of logit gradients exists at a time.  The reference repository has no joiner.
  *   h, rowinfo, grads, lse, dlogits  point at the block's first row;  rowinfo, grads, lse as
  *   written by cwr_joint_forward;  w, bias, dtype, H, V, N, blank as there;
+ *   dlogits  aligned to 16 bytes when V is a multiple of 8 (rows then leave as 16-byte stores), to
+ *            8 bytes when V is a multiple of 4, else to its element size;
  *   grad_costs, grad_stride, grad_scale as for cwr_backward. */
 int cwr_joint_backward(const void* h, const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
                        int64_t N, int32_t blank, const int32_t* rowinfo, const float* grads, const float* lse,

@@ -13,13 +13,17 @@ from compactwarprnntloss_amd import _lib
 from oracle import rnnt_oracle as orc
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "cwarp_rnnt_hip.h")
+HEADERS = [os.path.join(ROOT, "include", f) for f in sorted(os.listdir(os.path.join(ROOT, "include"))) if f.endswith(".h")]
 
 
 def declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(cwr_[a-z_0-9]+)\s*\(", text)))
+    """Every function any header under include/ declares (the drop-in surface and the test hooks)."""
+    names = set()
+    for header in HEADERS:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(cwr_[a-z_0-9]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -121,6 +125,18 @@ def test_invalid_calls_are_rejected_on_the_host():
     assert fwd(x=p(1) + 2) == 6         # CWR_ERR_ALIGN
     assert fwd(ws=p(5) + 8) == 6
     assert fwd(N=1 << 31) == 8          # CWR_ERR_TOO_LARGE
+
+    # the entry point that allocates nothing judges the same things before it looks its scratch up
+    def noalloc(**kw):
+        a = dict(ok_args, **kw)
+        return lib.cwr_forward_noalloc(a["x"], a["dtype"], a["R"], a["V"], a["lx"], a["ly"], a["y"], a["y_stride"],
+                                       a["y_len"], a["N"], a["blank"], a["mode"], a["max_u"], a["row_off"],
+                                       a["lab_off"], a["status"], a["rowinfo"], a["lse"], a["grads"], a["costs"],
+                                       a["stream"])
+
+    assert noalloc(costs=None) == 1 and noalloc(rowinfo=None) == 1 and noalloc(status=None) == 1
+    assert noalloc(grads=p(11) + 4) == 6 and noalloc(row_off=p(6) + 4) == 6
+    assert noalloc(blank=8) == 5 and noalloc(max_u=-1) == 4
 
     assert lib.cwr_offsets(None, None, 3, 10, p(1), p(2), p(3), None) == 1
     assert lib.cwr_offsets(p(1), p(2), -3, 10, p(1), p(2), p(3), None) == 4
@@ -288,6 +304,8 @@ def test_joint_entry_points_reject_invalid_calls_on_the_host():
         assert bwd(**{name: None}) == 1, name
     assert bwd(h=A + 8) == 6 and bwd(ri=A + 4) == 6 and bwd(dz=A + 4) == 6 and bwd(lse=A + 2) == 6
     assert bwd(V=41, dz=A + 1) == 6      # (rows off the 8-byte grid only need element alignment)
+    assert bwd(V=40, dz=A + 8) == 6      # rows of a multiple of 8 entries leave as 16-byte stores
+    assert bwd(V=44, dz=A + 4) == 6      # ... of a multiple of 4 as 8-byte stores
 
     def fwd(dtype=_lib.BF16, H=64, h=A, w=A):
         return lib.cwr_joint_forward(h, w, None, dtype, 100, H, 40, A, A, A, 3, 6, 2, 0, 3, A, 1 << 20, A, A, A, A, A, A,

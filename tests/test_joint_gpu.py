@@ -112,17 +112,20 @@ def test_joint_backward_dlogits_match_oracle(dtype, lx, ly, H, V, bias, blank):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
-@pytest.mark.parametrize("reduction", ["mean", "none"])
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
 def test_fused_joint_loss_gradients_match_oracle(dtype, reduction):
     """loss -> (dh, dW, dbias) through the autograd node, against the oracle's chain rule
-    (dense fused gradient of the float64 logits, then joint_backward).  The backward pass forms the
-    logits a block of rows at a time; a small block size makes the test cross several blocks.
-    Tolerance of the gradients: one rounding of d logits to the 16-bit type before the products."""
+    (dense fused gradient of the float64 logits, then joint_backward).  'mean' and 'sum' are the
+    node's own reductions (a scalar gradient comes back and the node spreads it, with 1/N for the
+    mean); 'none' weights the per-sequence costs by hand.  The backward pass forms the logits a block
+    of rows at a time; a small block size makes the test cross several blocks.  Tolerance of the
+    gradients: one rounding of d logits to the 16-bit type before the products."""
     import compactwarprnntloss_amd as pkg
     j = make_joint([40, 33, 17], [12, 20, 5], 96, 300 if dtype == "bf16" else 256, seed=9, dtype=dtype, scale=3.0)
     N = j["N"]
     w = np.random.default_rng(1).uniform(0.5, 1.5, N)
-    go = w / N if reduction == "mean" else w
+    c = 0.7
+    go = {"mean": np.full(N, c / N), "sum": np.full(N, c), "none": w}[reduction]
     z, ref = reference(j, grad_out=go, want_dense=True)
     dh_ref, dw_ref, db_ref = orc.joint_backward(ref["grad"], j["h"].double().numpy(), j["w"].double().numpy())
     h = j["h"].to(DEV).requires_grad_(True)
@@ -131,12 +134,13 @@ def test_fused_joint_loss_gradients_match_oracle(dtype, reduction):
     lx, ly = torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV)
     y = torch.from_numpy(j["yp"]).to(DEV)
     wt = torch.from_numpy(w).to(DEV).float()
-    if reduction == "mean":
-        # per-sequence weights through a mean: weight the costs by hand
-        costs = pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "none", chunk_rows=257)
-        loss = (costs * wt).mean()
-    else:
+    if reduction == "none":
         loss = (pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, "none", chunk_rows=257) * wt).sum()
+    else:
+        loss = pkg.fused_joint_loss(h, W, b, lx, y, ly, 0, reduction, chunk_rows=257) * c
+        _, ref0 = reference(j)
+        want = ref0["costs"].mean() if reduction == "mean" else ref0["costs"].sum()
+        assert abs(loss.item() / c - want) <= LOSS_RTOL * want
     loss.backward()
     torch.cuda.synchronize()
     rel = 1e-2 if dtype == "bf16" else 2e-3

@@ -375,3 +375,45 @@ def test_joint_layer_restatement_against_finite_differences_and_torch():
             dn = total(h, w, b)
             arr[idx] = keep
             assert abs((up - dn) / (2 * eps) - grad[idx]) < 1e-6, (idx, (up - dn) / (2 * eps), grad[idx])
+
+
+# ----------------------------------------------------------------------------- the C restatement
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("labels", ["2d", "1d"])
+def test_c_restatement_agrees_with_the_numpy_oracle(fused, labels):
+    """oracle/rnnt_oracle_c.c (the CPU baseline of the benchmark) against the NumPy oracle, which the
+    tests above pin: random ragged batches with U = 0, T = 1, labels that equal the blank, weights of
+    both signs; costs and sparse gradients to rounding of float64, dense gradients to the float32
+    they are stored in."""
+    from oracle import build_c
+    lib = build_c.load()
+    rng = np.random.default_rng(5 + fused)
+    for trial in range(6):
+        N = int(rng.integers(1, 7))
+        lx = rng.integers(1, 14, N).astype(np.int32)
+        ly = rng.integers(0, 9, N).astype(np.int32)
+        if trial == 0:
+            lx[0], ly[0] = 1, 0
+        V = int(rng.integers(2, 20))
+        blank = int(rng.integers(0, V))
+        R = int((lx.astype(np.int64) * (ly + 1)).sum())
+        x = (rng.standard_normal((R, V)) * 2).astype(np.float32)
+        if not fused:
+            x = orc.log_softmax(x).astype(np.float32)
+        yp = rng.integers(0, V, (N, max(int(ly.max()), 1))).astype(np.int32)  # may equal the blank
+        y = yp if labels == "2d" else np.concatenate([yp[n, : ly[n]] for n in range(N)]).astype(np.int32)
+        go = rng.uniform(-1.5, 1.5, N)
+        ref = orc.loss_and_grad(x.astype(np.float64), lx, y, ly, blank, "fused" if fused else "logprob", grad_out=go)
+        got = build_c.loss_and_grad(lib, x, lx, y, ly, blank, fused, go)
+        np.testing.assert_allclose(got["costs"], ref["costs"], rtol=1e-12)
+        np.testing.assert_allclose(got["G"], ref["G"], rtol=0, atol=1e-12)
+        np.testing.assert_allclose(got["grad"], ref["grad"], rtol=2e-7, atol=1e-9)
+    assert lib.rnnt_oracle_c_threads() >= 1
+
+
+def test_c_restatement_refuses_lengths_that_do_not_add_up():
+    from oracle import build_c
+    lib = build_c.load()
+    x = np.zeros((5, 3), dtype=np.float32)
+    with pytest.raises(RuntimeError):
+        build_c.loss_and_grad(lib, x, np.array([2], np.int32), np.zeros((1, 1), np.int32), np.array([1], np.int32))

@@ -253,6 +253,7 @@ def test_data_dependent_problems_are_flagged_not_faulted():
     b2c["yc"] = b["yc"][:-1].copy()
     out = run_device(b2c, True, labels="1d", max_u=3)
     assert out["flags"] & _lib.FLAG_BAD_LABEL and np.isnan(out["costs"][1]) and np.isfinite(out["costs"][0])
+    assert np.isfinite(out["G"]).all() and not out["G"][out["row_off"][1]:out["row_off"][2]].any()
     # lengths that claim more rows than x has
     b3 = dict(b)
     b3["lx"] = np.array([5, 60], dtype=np.int32)
@@ -289,6 +290,13 @@ def test_a_wait_that_runs_out_ends_the_walk_and_poisons_only_its_sequence():
             assert out["flags"] & _lib.FLAG_INTERNAL
             assert np.isnan(out["costs"][1])
             np.testing.assert_allclose(out["costs"][[0, 2]], ref["costs"][[0, 2]], rtol=LOSS_RTOL)
+            if with_grad:
+                # the poisoned sequence's gradients are zeros, not whatever its unfinished lattice held:
+                # a caller that masks the NaN cost with a zero weight must not get NaN * 0
+                a, e = out["row_off"][1], out["row_off"][2]
+                assert not out["G"][a:e].any() and np.isfinite(out["grad"]).all()
+                assert not out["grad"][a:e].any()
+                np.testing.assert_allclose(out["G"][:a], ref["G"][:a], rtol=0, atol=GRAD_ATOL)
     finally:
         lib.cwr_debug_wait_limit(0)
     out = run_device(b, True)
