@@ -59,6 +59,8 @@ SIGNATURES = {
     "cwr_unpack": (C.c_int, [_p, C.c_int, _i64, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _p]),
     "cwr_joint_forward": (C.c_int, [_p, _p, _p, C.c_int, _i64, _i64, _i64, _p, _p, _p, _i64, _i64, _i64, _i32, _i64,
                                     _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
+    "cwr_joint_forward_fg": (C.c_int, [_p, _p, C.c_int, _i64, _i64, _p, _p, _p, C.c_int, _i64, _i64, _i64, _p, _p, _p,
+                                       _i64, _i64, _i64, _i32, _i64, _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
     "cwr_joint_backward": (C.c_int, [_p, _p, _p, C.c_int, _i64, _i64, _i64, _i64, _i32, _p, _p, _p, _p, _i64, C.c_float,
                                      _p, _p]),
     "cwr_join": (C.c_int, [_p, _p, C.c_int, C.c_int, _i64, _i64, _i64, _i64, _p, _p, _p, _i64, _p, _p, _p]),

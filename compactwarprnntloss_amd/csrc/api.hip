@@ -355,6 +355,31 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
     if (misaligned(h, 16) || misaligned(w, 16) || misaligned(bias, 4)) return CWR_ERR_ALIGN;
     JointOperands j;
     j.h = h; j.w = w; j.bias = bias; j.H = H;
+    j.f = nullptr; j.g = nullptr; j.h_out = nullptr; j.act = 0; j.T_pad = 0; j.Up_pad = 0;
+    return forward_impl(nullptr, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, CWR_MODE_FUSED, max_u, workspace,
+                        workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream, true,
+                        &j);
+}
+
+int cwr_joint_forward_fg(const void* f, const void* g, int act, int64_t T_pad, int64_t Up_pad, void* h_out,
+                         const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                         const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                         int64_t N, int32_t blank, int64_t max_u, void* workspace, size_t workspace_bytes_,
+                         int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
+                         float* grads, float* costs, void* stream) {
+    if (dtype != CWR_F16 && dtype != CWR_BF16) return CWR_ERR_DTYPE;
+    if (act < CWR_ACT_NONE || act > CWR_ACT_RELU) return CWR_ERR_MODE;
+    // the joint sizes whose rows a wave keeps in registers
+    if (H != 256 && H != 384 && H != 512 && H != 640 && H != 768 && H != 1024) return CWR_ERR_SHAPE;
+    if (T_pad < 0 || Up_pad < 0) return CWR_ERR_SHAPE;
+    if (T_pad > 0x3fffffff || Up_pad > 0x3fffffff) return CWR_ERR_TOO_LARGE;
+    if (R > 0 && (!f || !g || !w)) return CWR_ERR_NULL;
+    if (R > 0 && (T_pad == 0 || Up_pad == 0)) return CWR_ERR_SHAPE;
+    if (misaligned(f, 16) || misaligned(g, 16) || misaligned(h_out, 16) || misaligned(w, 16) || misaligned(bias, 4))
+        return CWR_ERR_ALIGN;
+    JointOperands j;
+    j.h = nullptr; j.w = w; j.bias = bias; j.H = H;
+    j.f = f; j.g = g; j.h_out = h_out; j.act = act; j.T_pad = T_pad; j.Up_pad = Up_pad;
     return forward_impl(nullptr, dtype, R, V, lx, ly, y, y_stride, y_len, N, blank, CWR_MODE_FUSED, max_u, workspace,
                         workspace_bytes_, row_off, lab_off, status, rowinfo, lse, grads, costs, nullptr, stream, true,
                         &j);

@@ -70,6 +70,13 @@ struct JointOperands {
     const void* w;
     const float* bias;  // may be null
     i64 H;
+    // h == null: the joint rows are formed in the kernel, row(n,t,u) = act(f[n,t,:] + g[n,u,:]), from
+    // f (N,T_pad,H) and g (N,Up_pad,H); h_out (may be null) receives them
+    const void* f;
+    const void* g;
+    void* h_out;
+    int act;
+    i64 T_pad, Up_pad;
 };
 int launch_joint_gather(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,
                         float* grads);

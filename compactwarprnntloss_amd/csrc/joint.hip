@@ -26,6 +26,7 @@
 //              vocabulary in tiles of 128, both operand tiles through LDS in K-slices of 32; waves
 //              split the tile 2 x 2: wave (wd, wv) multiplies the data rows [128 wd, 128 wd + 128)
 //              with the vocabulary entries [64 wv, 64 wv + 64) of the tile.
+#include "cwr_act.hpp"
 #include "cwr_device.hpp"
 #include "cwr_host.hpp"
 
@@ -614,6 +615,78 @@ __device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 
     }
 }
 
+// The same fragments formed on the spot from the joiner's two inputs, row(n,t,u) = act(f[n,t,:] +
+// g[n,u,:]) (the arithmetic of the join kernels: sum and activation in fp32, one rounding to the
+// 16-bit type), for callers that never want the (R,H) joint rows in memory: f and g are a few MB and
+// come out of the L2.  h_out (may be null) receives the rows for a backward pass that needs them.
+template <typename T> struct JoinSrc {
+    const T* f;
+    const T* g;
+    T* h_out;
+    int act;
+    int T_pad, Up_pad;
+    const int* lx;
+    const int* ly;
+    const i64* row_off;
+    int N;
+    int* status;
+};
+
+template <typename T, int ACT, int ND, int KS>
+__device__ __forceinline__ void join_resident_rows_as(const JoinSrc<T>& s, i64 R, i64 row0, v4i (&hreg)[ND][KS]) {
+    constexpr int H = KS * 16;
+    const int lane = threadIdx.x & 63;
+    const int hf = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int nd = 0; nd < ND; ++nd) {
+        const i64 r = row0 + 32 * nd + l32;
+        const RowInfo ri = decode_row(r < R ? r : R - 1, R, s.row_off, s.lx, s.ly, s.N);
+        const bool ok = ri.n >= 0 && ri.t < s.T_pad && ri.u < s.Up_pad;
+        if (ri.n >= 0 && !ok) raise_flag(s.status, CWR_FLAG_BAD_LENGTH);  // the cell lies outside the padded inputs
+        // a row no valid cell maps to is a row of zeros, as in the join kernels
+        const T* pf = s.f + (ok ? ((i64)ri.n * s.T_pad + ri.t) * H : 0) + 8 * hf;
+        const T* pg = s.g + (ok ? ((i64)ri.n * s.Up_pad + ri.u) * H : 0) + 8 * hf;
+        T* po = (s.h_out && r < R) ? s.h_out + r * (i64)H + 8 * hf : nullptr;
+        // All of f's fragments are requested at once, straight into the registers the row will live
+        // in; g's follow in batches of kBatch into spare registers and each batch is folded in as it
+        // arrives.  (One fragment of each at a time, which is what the loop would otherwise compile
+        // to, pays a trip to the L2 per fragment: 32 of them in a row at H = 512.)
+        constexpr int kBatch = KS >= 24 ? 4 : 8;  // the longer the resident row, the fewer spare registers
+        static_assert(KS % kBatch == 0, "whole batches");
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) hreg[nd][ks] = *reinterpret_cast<const v4i*>(pf + 16 * ks);
+#pragma unroll
+        for (int k0 = 0; k0 < KS; k0 += kBatch) {
+            v4i gq[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) gq[i] = *reinterpret_cast<const v4i*>(pg + 16 * (k0 + i));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                PackT<T, 8> a, b, o;
+                __builtin_memcpy(&a, &hreg[nd][k0 + i], 16);
+                __builtin_memcpy(&b, &gq[i], 16);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    o.e[e] = ok ? Arith<T>::down(activate<ACT, T>(Arith<T>::up(a.e[e]) + Arith<T>::up(b.e[e])))
+                                : Arith<T>::down(0.f);
+                v4i v;
+                __builtin_memcpy(&v, &o, 16);
+                hreg[nd][k0 + i] = v;
+                if (po) *reinterpret_cast<v4i*>(po + 16 * (k0 + i)) = v;
+                __builtin_amdgcn_sched_barrier(0);  // one fragment's temporaries at a time
+            }
+        }
+    }
+}
+
+template <typename T, int ND, int KS>
+__device__ __forceinline__ void join_resident_rows(const JoinSrc<T>& s, i64 R, i64 row0, v4i (&hreg)[ND][KS]) {
+    if (s.act == kActTanh) join_resident_rows_as<T, kActTanh, ND, KS>(s, R, row0, hreg);
+    else if (s.act == kActRelu) join_resident_rows_as<T, kActRelu, ND, KS>(s, R, row0, hreg);
+    else join_resident_rows_as<T, kActNone, ND, KS>(s, R, row0, hreg);
+}
+
 // tile(acc, v0) receives acc[mv][nd] = vocabulary entries [v0 + 32 mv, v0 + 32 mv + 32) x data rows
 // [row0 + 32 nd, row0 + 32 nd + 32) of this wave; the vocabulary is walked in tiles of JN = 32 NMV.
 // Order of the start-up, which every workgroup of a round runs at the same time as every other: the
@@ -621,8 +694,9 @@ __device__ __forceinline__ void load_resident_rows(const T* __restrict__ h, i64 
 // (what the caller still has to do about its rows: loads issued here queue up BEHIND the rows',
 // whatever the caller asked for earlier is served before them), and the first tile starts as
 // soon as the first fragments are there.
-template <typename T, int ND, int KS, int NMV, int WAVES, int RK, bool D2, typename AfterIssue, typename TileFn>
-__device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i64 row0, const T* __restrict__ W,
+template <typename T, int ND, int KS, int NMV, int WAVES, int RK, bool D2, typename LoadRows, typename AfterIssue,
+          typename TileFn>
+__device__ __forceinline__ void walk_resident(LoadRows&& load_rows, const T* __restrict__ W,
                                               const float* __restrict__ bias, int V, ResLds<T, NMV, RK>& lds,
                                               AfterIssue&& after_issue, TileFn&& tile) {
     constexpr int JN = 32 * NMV;
@@ -669,7 +743,7 @@ __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i6
     float bias_next = 0.f;
     if (tid < JN) s_bias[0][tid] = bias_of(0);
     v4i hreg[ND][KS];
-    load_resident_rows<T, ND, KS>(h, R, row0, hreg);
+    load_rows(hreg);
     after_issue();
     fetch(0, 0, pre[0]);
     if (D2 && (NK > 1 || nvt > 1)) fetch(NK > 1 ? 0 : 1, NK > 1 ? 1 : 0, pre[1]);
@@ -738,9 +812,9 @@ __device__ __forceinline__ void walk_resident(const T* __restrict__ h, i64 R, i6
     for (int vt = 1; vt < nvt; ++vt) one_tile(vt);
 }
 
-template <typename T, int ND, int KS, int NMV, int WAVES, int RK, int OCC, bool D2>
+template <typename T, int ND, int KS, int NMV, int WAVES, int RK, int OCC, bool D2, bool FG>
 __global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_fwd_res(
-    const T* __restrict__ h, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
+    const T* __restrict__ h, const JoinSrc<T> js, const T* __restrict__ W, const float* __restrict__ bias, i64 R, int V,
     const int* __restrict__ lx, const int* __restrict__ ly, const int* __restrict__ y, i64 y_stride, i64 y_len,
     const i64* __restrict__ row_off, const i64* __restrict__ lab_off, const i64* __restrict__ pad_off, int N,
     int blank, const FwdOut out, int* __restrict__ status) {
@@ -754,7 +828,11 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_fwd_res(
                                            status);
     fwd_rows_finish<ND>(q, tb, row0, row0 + l32, R, y, y_stride, y_len, N, V, status);
     walk_resident<T, ND, KS, NMV, WAVES, RK, D2>(
-        h, R, row0, W, bias, V, lds, [&]() {},
+        [&](v4i (&hreg)[ND][KS]) {
+            if (FG) join_resident_rows<T, ND, KS>(js, R, row0, hreg);
+            else load_resident_rows<T, ND, KS>(h, R, row0, hreg);
+        },
+        W, bias, V, lds, [&]() {},
         [&](const f32x16 (&acc)[NMV][ND], int v0) { fwd_fold_tile<NMV, ND>(acc, v0, blank, hf, q); });
     fwd_merge_halves<ND>(q);
 #pragma unroll
@@ -781,7 +859,8 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_dz_res(
     DzRaw<ND> raw;
     dz_rows_begin<ND>(raw, row0 + l32, R, rowinfo, grads, lse);
     walk_resident<T, ND, KS, NMV, WAVES, RK, D2>(
-        h, R, row0, W, bias, V, lds, [&]() { dz_rows_finish<ND>(q, raw, row0 + l32, R, N, go); },
+        [&](v4i (&hreg)[ND][KS]) { load_resident_rows<T, ND, KS>(h, R, row0, hreg); }, W, bias, V, lds,
+        [&]() { dz_rows_finish<ND>(q, raw, row0 + l32, R, N, go); },
         [&](const f32x16 (&acc)[NMV][ND], int v0) {
             dz_store_tile<T, NMV, ND>(acc, v0, V, blank, hf, row0 + l32, row0 + 32 * ND, R, q, dz, tbuf);
         });
@@ -812,17 +891,28 @@ static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOp
     const FwdOut out = {ws.lp, lse, reinterpret_cast<int2*>(rowinfo), reinterpret_cast<float2*>(grads), ws.seqmode};
     const T* h = static_cast<const T*>(j.h);
     const T* w = static_cast<const T*>(j.w);
-#define CWR_JOINT_RES(ND, KS, NMV, WAVES, RK, OCC, D2)                                                                           \
-    if (j.H == 16 * KS) {                                                                                        \
-        const i64 blocks = (b.R + 32 * ND * WAVES - 1) / (32 * ND * WAVES);                                                  \
-        if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                     \
-        CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, WAVES, RK, OCC, D2>), dim3((unsigned)blocks), dim3(64 * WAVES), 0, b.stream, h, w,  \
-                   j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride, b.y_len, b.row_off, b.lab_off, ws.pad_off,     \
-                   b.N, b.blank, out, b.status);                                                                 \
-        return check_launch();                                                                                   \
+    JoinSrc<T> js;
+    js.f = static_cast<const T*>(j.f); js.g = static_cast<const T*>(j.g); js.h_out = static_cast<T*>(j.h_out);
+    js.act = j.act; js.T_pad = (int)j.T_pad; js.Up_pad = (int)j.Up_pad;
+    js.lx = b.lx; js.ly = b.ly; js.row_off = b.row_off; js.N = b.N; js.status = b.status;
+    const bool fg = j.h == nullptr;
+#define CWR_JOINT_RES(ND, KS, NMV, WAVES, RK, OCC, D2)                                                            \
+    if (j.H == 16 * KS) {                                                                                         \
+        const i64 blocks = (b.R + 32 * ND * WAVES - 1) / (32 * ND * WAVES);                                       \
+        if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;                                                      \
+        if (fg)                                                                                                   \
+            CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, WAVES, RK, OCC, D2, true>), dim3((unsigned)blocks),       \
+                       dim3(64 * WAVES), 0, b.stream, h, js, w, j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride,    \
+                       b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, out, b.status);                   \
+        else                                                                                                      \
+            CWR_LAUNCH((k_joint_fwd_res<T, ND, KS, NMV, WAVES, RK, OCC, D2, false>), dim3((unsigned)blocks),      \
+                       dim3(64 * WAVES), 0, b.stream, h, js, w, j.bias, b.R, b.V, b.lx, b.ly, b.y, b.y_stride,    \
+                       b.y_len, b.row_off, b.lab_off, ws.pad_off, b.N, b.blank, out, b.status);                   \
+        return check_launch();                                                                                    \
     }
     CWR_JOINT_SHAPES(CWR_JOINT_RES)
 #undef CWR_JOINT_RES
+    if (fg) return CWR_ERR_SHAPE;  // the rows are formed in registers: resident joint sizes only
     const i64 blocks = (b.R + kJM - 1) / kJM;
     if (blocks > 0x7fffffffLL) return CWR_ERR_TOO_LARGE;
     CWR_LAUNCH((k_joint_fwd<T>), dim3((unsigned)blocks), dim3(256), 0, b.stream, h, w, j.bias, b.R, (int)j.H, b.V,

@@ -13,7 +13,8 @@ from typing import Any, Optional
 import torch
 
 from . import _lib
-from .loss import _DTYPES, _offsets, _raise_on_flags, _raise_on_status, _stream_ptr, joint_forward
+from .loss import (RESIDENT_JOINT_SIZES, _DTYPES, _offsets, _raise_on_flags, _raise_on_status, _stream_ptr,
+                   joint_forward, joint_forward_fg)
 
 _ACTS = {None: 0, "none": 0, "tanh": 1, "relu": 2}
 _DW_SPLIT = 16  # parts the rows of a block are cut into for the weight-gradient product
@@ -114,49 +115,137 @@ class _JointLoss(torch.autograd.Function):
     @staticmethod
     def backward(ctx: Any, grad_out):
         h, weight, bias, lx, ys, ly = ctx.saved_tensors
+        dh, dw, db = _joint_backward(h, weight, bias if ctx.has_bias else None, ctx.state, grad_out, ctx.reduction,
+                                     ctx.blank, ctx.chunk_rows)
+        return dh, dw, db, None, None, None, None, None, None, None, None
+
+
+def _joint_backward(h, weight, bias, st, grad_out, reduction, blank, chunk_rows):
+    """(dh, dW, dbias) of the loss of logits = h @ weight.T + bias from the state its forward call left:
+    cwr_joint_backward a block of rows at a time, library GEMMs on each block."""
+    lib = _lib.load()
+    dev = h.device
+    R, H = h.shape
+    V = weight.size(0)
+    N = st.N
+    gc = grad_out.to(torch.float32).reshape(-1)
+    if gc.numel() == 1:
+        gc = gc.expand(N)
+    gc = (gc / N if reduction == "mean" else gc).contiguous()
+    dh = torch.empty_like(h)
+    dw = torch.zeros((V, H), dtype=torch.float32, device=dev)
+    db = torch.zeros(V, dtype=torch.float32, device=dev) if bias is not None else None
+    bias_f = bias.to(torch.float32).contiguous() if bias is not None else None
+    chunk = max(1, min(int(chunk_rows), R))
+    z = torch.empty((chunk, V), dtype=h.dtype, device=dev)
+    with torch.cuda.device(dev):
+        stream = _stream_ptr(dev)
+        for r0 in range(0, R, chunk):
+            r1 = min(R, r0 + chunk)
+            zc = z[: r1 - r0]
+            rc = lib.cwr_joint_backward(h[r0:].data_ptr(), weight.data_ptr(),
+                                        bias_f.data_ptr() if bias_f is not None else None, _DTYPES[h.dtype],
+                                        r1 - r0, H, V, N, int(blank), st.rowinfo[r0:].data_ptr(),
+                                        st.grads[r0:].data_ptr(), st.lse[r0:].data_ptr(), gc.data_ptr(), 1, 1.0,
+                                        zc.data_ptr(), stream)
+            _lib.check(rc, "cwr_joint_backward")
+            torch.mm(zc, weight, out=dh[r0:r1])
+            # dW += zc^T h[r0:r1].  The contraction runs over the rows, the result is only (V, H): as one
+            # GEMM the library fills a quarter of the GPU with it, so the rows are cut into _DW_SPLIT
+            # parts multiplied as a batch (16-bit products of a part each, summed in fp32)
+            n = r1 - r0
+            m = (n // _DW_SPLIT) * _DW_SPLIT
+            if m:
+                part = torch.bmm(zc[:m].view(_DW_SPLIT, m // _DW_SPLIT, V).transpose(1, 2),
+                                 h[r0:r0 + m].view(_DW_SPLIT, m // _DW_SPLIT, H))
+                dw.add_(part.sum(dim=0, dtype=torch.float32))
+            if n > m:
+                dw.add_(torch.mm(zc[m:n].t(), h[r0 + m:r1]))
+            if db is not None:
+                db.add_(zc.sum(dim=0, dtype=torch.float32))
+    dbias = db.to(bias.dtype) if db is not None else None
+    return dh, dw.to(weight.dtype), dbias
+
+
+class _JoinerLoss(torch.autograd.Function):
+    """The whole joiner behind the loss: rows act(f[n,t] + g[n,u]) formed inside the output-layer kernel
+    (cwr_joint_forward_fg).  When nothing asks for a gradient the (R, H) rows never exist; otherwise
+    the kernel leaves them behind for the backward pass (logit gradients, weight-gradient product,
+    cwr_join_backward)."""
+
+    @staticmethod
+    def forward(ctx: Any, f, g, weight, bias, lx, ys, ly, blank, reduction, act, total_rows, max_u, validate,
+                chunk_rows):
+        need = any(ctx.needs_input_grad[:4])
+        costs, st, h = joint_forward_fg(f, g, act, weight, bias, lx, ys, ly, blank, total_rows, max_u, keep_rows=need)
+        if validate:
+            _raise_on_flags(st)
+        st.workspace = None
+        ctx.state = st
+        ctx.blank, ctx.reduction, ctx.chunk_rows, ctx.act = blank, reduction, int(chunk_rows), act
+        ctx.dims = (f.size(0), f.size(1), g.size(1), f.size(2))
+        ctx.has_bias = bias is not None
+        if need:
+            ctx.save_for_backward(h, weight, bias if bias is not None else f.new_empty(0), lx, ly)
+        if reduction == "mean":
+            return costs.mean()
+        if reduction == "sum":
+            return costs.sum()
+        return costs
+
+    @staticmethod
+    def backward(ctx: Any, grad_out):
+        h, weight, bias, lx, ly = ctx.saved_tensors
         st = ctx.state
+        dh, dw, db = _joint_backward(h, weight, bias if ctx.has_bias else None, st, grad_out, ctx.reduction,
+                                     ctx.blank, ctx.chunk_rows)
+        N, T, Up, H = ctx.dims
         lib = _lib.load()
-        dev = h.device
-        R, H = h.shape
-        V = weight.size(0)
-        N = st.N
-        gc = grad_out.to(torch.float32).reshape(-1)
-        if gc.numel() == 1:
-            gc = gc.expand(N)
-        gc = (gc / N if ctx.reduction == "mean" else gc).contiguous()
-        dh = torch.empty_like(h)
-        dw = torch.zeros((V, H), dtype=torch.float32, device=dev)
-        db = torch.zeros(V, dtype=torch.float32, device=dev) if ctx.has_bias else None
-        bias_f = bias.to(torch.float32).contiguous() if ctx.has_bias else None
-        chunk = max(1, min(ctx.chunk_rows, R))
-        z = torch.empty((chunk, V), dtype=h.dtype, device=dev)
-        with torch.cuda.device(dev):
-            stream = _stream_ptr(dev)
-            for r0 in range(0, R, chunk):
-                r1 = min(R, r0 + chunk)
-                zc = z[: r1 - r0]
-                rc = lib.cwr_joint_backward(h[r0:].data_ptr(), weight.data_ptr(),
-                                            bias_f.data_ptr() if bias_f is not None else None, _DTYPES[h.dtype],
-                                            r1 - r0, H, V, N, int(ctx.blank), st.rowinfo[r0:].data_ptr(),
-                                            st.grads[r0:].data_ptr(), st.lse[r0:].data_ptr(), gc.data_ptr(), 1, 1.0,
-                                            zc.data_ptr(), stream)
-                _lib.check(rc, "cwr_joint_backward")
-                torch.mm(zc, weight, out=dh[r0:r1])
-                # dW += zc^T h[r0:r1].  The contraction runs over the rows, the result is only (V, H): as one
-                # GEMM the library fills a quarter of the GPU with it, so the rows are cut into _DW_SPLIT
-                # parts multiplied as a batch (16-bit products of a part each, summed in fp32)
-                n = r1 - r0
-                m = (n // _DW_SPLIT) * _DW_SPLIT
-                if m:
-                    part = torch.bmm(zc[:m].view(_DW_SPLIT, m // _DW_SPLIT, V).transpose(1, 2),
-                                     h[r0:r0 + m].view(_DW_SPLIT, m // _DW_SPLIT, H))
-                    dw.add_(part.sum(dim=0, dtype=torch.float32))
-                if n > m:
-                    dw.add_(torch.mm(zc[m:n].t(), h[r0 + m:r1]))
-                if db is not None:
-                    db.add_(zc.sum(dim=0, dtype=torch.float32))
-        dbias = db.to(bias.dtype) if db is not None else None
-        return dh, dw.to(weight.dtype), dbias, None, None, None, None, None, None, None, None
+        df = torch.empty((N, T, H), dtype=dh.dtype, device=dh.device)
+        dg = torch.empty((N, Up, H), dtype=dh.dtype, device=dh.device)
+        with torch.cuda.device(dh.device):
+            rc = lib.cwr_join_backward(dh.data_ptr(), h.data_ptr() if ctx.act else None, _DTYPES[dh.dtype], ctx.act,
+                                       N, T, Up, H, lx.data_ptr(), ly.data_ptr(), st.row_off.data_ptr(), dh.size(0),
+                                       df.data_ptr(), dg.data_ptr(), _stream_ptr(dh.device))
+            _lib.check(rc, "cwr_join_backward")
+        return df, dg, dw, db, None, None, None, None, None, None, None, None, None, None
+
+
+def fused_joiner_loss(f: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                      lx: torch.Tensor, y: torch.Tensor, ly: torch.Tensor, blank: int = 0,
+                      reduction: Optional[str] = "mean", activation: Optional[str] = "tanh", *,
+                      total_rows: Optional[int] = None, max_u: Optional[int] = None, validate: bool = False,
+                      chunk_rows: int = 131072, one_kernel: Optional[bool] = None) -> torch.Tensor:
+    """transducer_loss of the logits act(f[n,t] + g[n,u]) @ weight.T + bias, the joiner's whole chain,
+    with neither the (R, H) joint rows nor the (R, V) logits in memory on the way to the loss: f
+    (N, T, H) encoder frames and g (N, U+1, H) predictor states projected to the joint space, weight
+    (V, H) and bias (V,) or None the output layer, fp16 or bf16.  Differentiable in f, g, weight and
+    bias (the backward pass does hold the joint rows and chunk_rows x V logit gradients).
+
+    one_kernel: True forms the joint rows inside the output-layer kernel (cwr_joint_forward_fg; joint
+    sizes in RESIDENT_JOINT_SIZES only), False runs compact_join and fused_joint_loss one after the
+    other, None picks by speed: the one-kernel form wins up to H = 384 (N=32, V=1024, H=256, bf16:
+    forward 0.28 against 0.31 ms) and loses beyond (H=512: 0.53 against 0.46 ms: every wave of the GPU
+    forms its rows at the same moment, with no matrix work of another wave to hide behind), where it
+    remains the choice of a caller who cannot afford the (R, H) rows in memory."""
+    if activation not in _ACTS:
+        raise RuntimeError(f"activation must be one of {sorted(k for k in _ACTS if k)} or None")
+    assert lx.dtype == torch.int32 and ly.dtype == torch.int32 and y.dtype == torch.int32
+    assert reduction in ["mean", "sum", "none"] or reduction is None
+    assert blank >= 0 and blank < weight.size(0)
+    if total_rows is None:
+        total_rows = int((lx.long() * (ly.long() + 1)).sum().item())
+    if one_kernel is None:
+        one_kernel = f.size(-1) in RESIDENT_JOINT_SIZES and f.size(-1) <= 384
+    if one_kernel and f.size(-1) not in RESIDENT_JOINT_SIZES:
+        raise RuntimeError(f"one_kernel needs a joint dimension in {RESIDENT_JOINT_SIZES}")
+    if not one_kernel:
+        h = compact_join(f, g, lx, ly, activation, total_rows, validate)
+        return fused_joint_loss(h, weight, bias, lx, y, ly, blank, reduction, max_u=max_u, validate=validate,
+                                chunk_rows=chunk_rows)
+    return _JoinerLoss.apply(f.contiguous(), g.contiguous(), weight.contiguous(), bias, lx, y, ly, int(blank),
+                             reduction if reduction in ("mean", "sum") else "none", _ACTS[activation],
+                             int(total_rows), max_u, bool(validate), int(chunk_rows))
 
 
 def fused_joint_loss(h: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], lx: torch.Tensor,
@@ -193,7 +282,8 @@ class CompactJoiner(torch.nn.Module):
 
     def loss(self, enc_out, pred_out, lx, y, ly, blank: int = 0, reduction: Optional[str] = "mean",
              total_rows: Optional[int] = None):
-        """The transducer loss of this joiner's logits without storing them (fp16 / bf16 modules):
-        compact_join, then fused_joint_loss on the output layer's weight and bias."""
-        h = compact_join(self.enc(enc_out), self.pred(pred_out), lx, ly, self.activation, total_rows)
-        return fused_joint_loss(h, self.out.weight, self.out.bias, lx, y, ly, blank, reduction)
+        """The transducer loss of this joiner's logits without storing them (fp16 / bf16 modules): the
+        broadcast sum, the activation and the output layer all run inside the loss's own kernel
+        (fused_joiner_loss)."""
+        return fused_joiner_loss(self.enc(enc_out), self.pred(pred_out), self.out.weight, self.out.bias, lx, y, ly,
+                                 blank, reduction, self.activation, total_rows=total_rows)

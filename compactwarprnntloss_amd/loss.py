@@ -116,25 +116,23 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     return costs, st
 
 
-def joint_forward(h, weight, bias, lx, ys, ly, blank: int, max_u: Optional[int] = None):
-    """Binding of cwr_joint_forward: the loss of logits = h @ weight.T + bias without ever storing
-    them.  h (R,H) and weight (V,H) fp16 or bf16, bias (V,) or None.  Returns (costs fp32 (N,),
-    ForwardState) like rnnt_forward in fused mode."""
-    if h.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != h.dtype:
-        raise RuntimeError("h and weight must both be float16 or both bfloat16")
-    if h.dim() != 2 or weight.dim() != 2 or h.size(1) != weight.size(1):
-        raise RuntimeError("h must be (R, H) and weight (V, H)")
-    if h.size(1) % 32 != 0:
+RESIDENT_JOINT_SIZES = (256, 384, 512, 640, 768, 1024)  # joint sizes whose rows a wave keeps in registers
+
+
+def _joint_state(like, weight, bias, lx, ys, ly, R: int, max_u: Optional[int]):
+    """Checks and allocations shared by the two joint_forward bindings."""
+    if like.dtype not in (torch.float16, torch.bfloat16) or weight.dtype != like.dtype:
+        raise RuntimeError("the joint rows (or f and g) and weight must all be float16 or all bfloat16")
+    if weight.dim() != 2 or like.size(-1) != weight.size(1):
+        raise RuntimeError("weight must be (V, H) with the joint dimension H of the rows")
+    if like.size(-1) % 32 != 0:
         raise RuntimeError("the joint dimension must be a multiple of 32")
     if not weight.is_cuda or not weight.is_contiguous():
         raise RuntimeError("weight must be a contiguous CUDA tensor")
-    _check_inputs(h, lx, ys, ly)
     lib = _lib.load()
-    dev = h.device
+    dev = like.device
     N = lx.numel()
-    R, H = h.shape
     V = weight.size(0)
-    y_stride, y_len = _label_args(ys)
     if max_u is None:
         max_u = ys.size(1) if ys.dim() == 2 else (int(ly.max().item()) if ly.numel() else 0)
     b32 = None
@@ -155,15 +153,66 @@ def joint_forward(h, weight, bias, lx, ys, ly, blank: int, max_u: Optional[int] 
     st.lse = torch.empty(R, dtype=torch.float32, device=dev)
     st.grads = torch.empty((R, 2), dtype=torch.float32, device=dev)
     st.rowinfo = torch.empty((R, 2), dtype=torch.int32, device=dev)
+    return lib, st, costs, b32, ws_bytes
+
+
+def joint_forward(h, weight, bias, lx, ys, ly, blank: int, max_u: Optional[int] = None):
+    """Binding of cwr_joint_forward: the loss of logits = h @ weight.T + bias without ever storing
+    them.  h (R,H) and weight (V,H) fp16 or bf16, bias (V,) or None.  Returns (costs fp32 (N,),
+    ForwardState) like rnnt_forward in fused mode."""
+    if h.dim() != 2:
+        raise RuntimeError("h must be (R, H)")
+    _check_inputs(h, lx, ys, ly)
+    R, H = h.shape
+    lib, st, costs, b32, ws_bytes = _joint_state(h, weight, bias, lx, ys, ly, R, max_u)
+    dev = h.device
+    V, N = st.V, st.N
+    y_stride, y_len = _label_args(ys)
     with torch.cuda.device(dev):
         rc = lib.cwr_joint_forward(h.data_ptr(), weight.data_ptr(), b32.data_ptr() if b32 is not None else None,
                                    _DTYPES[h.dtype], R, H, V, lx.data_ptr(), ly.data_ptr(), ys.data_ptr(), y_stride,
-                                   y_len, N, int(blank), int(max_u), st.workspace.data_ptr(), ws_bytes,
+                                   y_len, N, int(blank), st.max_u, st.workspace.data_ptr(), ws_bytes,
                                    st.row_off.data_ptr(), st.lab_off.data_ptr(), st.status.data_ptr(),
                                    st.rowinfo.data_ptr(), st.lse.data_ptr(), st.grads.data_ptr(), costs.data_ptr(),
                                    _stream_ptr(dev))
         _lib.check(rc, "cwr_joint_forward")
     return costs, st
+
+
+def joint_forward_fg(f, g, act: int, weight, bias, lx, ys, ly, blank: int, total_rows: int,
+                     max_u: Optional[int] = None, keep_rows: bool = False):
+    """Binding of cwr_joint_forward_fg: the loss of logits = act(f[n,t] + g[n,u]) @ weight.T + bias
+    with the joint rows formed inside the kernel.  f (N,T,H), g (N,U+1,H), weight (V,H) fp16 or bf16;
+    act 0 / 1 / 2 = none / tanh / relu; H one of RESIDENT_JOINT_SIZES.  Returns (costs, ForwardState,
+    h): h the (R,H) joint rows when keep_rows, else None."""
+    if f.dim() != 3 or g.dim() != 3 or f.size(0) != g.size(0) or f.size(2) != g.size(2) or f.dtype != g.dtype:
+        raise RuntimeError("f must be (N, T, H) and g (N, U+1, H) of one dtype")
+    for name, t in (("f", f), ("g", g), ("lx", lx), ("ly", ly), ("y", ys)):
+        if not t.is_cuda or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous CUDA tensor")
+    if lx.dtype != torch.int32 or ly.dtype != torch.int32 or ys.dtype != torch.int32:
+        raise RuntimeError("lx, ly and y must be int32")
+    if lx.numel() != f.size(0) or ly.numel() != f.size(0):
+        raise RuntimeError("lx, ly must hold one entry per sequence")
+    H = f.size(2)
+    if H not in RESIDENT_JOINT_SIZES:
+        raise RuntimeError(f"joint dimension {H} not in {RESIDENT_JOINT_SIZES}: use compact_join + joint_forward")
+    R = int(total_rows)
+    lib, st, costs, b32, ws_bytes = _joint_state(f, weight, bias, lx, ys, ly, R, max_u)
+    dev = f.device
+    V, N = st.V, st.N
+    y_stride, y_len = _label_args(ys)
+    h = torch.empty((R, H), dtype=f.dtype, device=dev) if keep_rows else None
+    with torch.cuda.device(dev):
+        rc = lib.cwr_joint_forward_fg(f.data_ptr(), g.data_ptr(), int(act), f.size(1), g.size(1),
+                                      h.data_ptr() if h is not None else None, weight.data_ptr(),
+                                      b32.data_ptr() if b32 is not None else None, _DTYPES[f.dtype], R, H, V,
+                                      lx.data_ptr(), ly.data_ptr(), ys.data_ptr(), y_stride, y_len, N, int(blank),
+                                      st.max_u, st.workspace.data_ptr(), ws_bytes, st.row_off.data_ptr(),
+                                      st.lab_off.data_ptr(), st.status.data_ptr(), st.rowinfo.data_ptr(),
+                                      st.lse.data_ptr(), st.grads.data_ptr(), costs.data_ptr(), _stream_ptr(dev))
+        _lib.check(rc, "cwr_joint_forward_fg")
+    return costs, st, h
 
 
 def rnnt_backward(xs, lx, ys, ly, blank: int, st: ForwardState, grad_costs: torch.Tensor,

@@ -293,6 +293,26 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
                       int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
                       float* grads, float* costs, void* stream);
 
+/* cwr_joint_forward with the joint rows formed inside the kernel: the whole chain of the joiner,
+ * h[row(n,t,u), :] = act(f[n,t,:] + g[n,u,:]) (cwr_join's arithmetic: sum and activation in fp32, one
+ * rounding to `dtype`), output layer, log-softmax and gather, as ONE kernel behind the loss.  f and g
+ * are a few MB and are served by the L2; neither the (R, H) joint rows nor the (R, V) logits have to
+ * exist in memory.  The reference repository has no joiner (see cwr_join).
+ *   f (N, T_pad, H), g (N, Up_pad, H), w (V, H) of `dtype` = CWR_F16 or CWR_BF16, contiguous, 16-byte
+ *         aligned;  act a cwr_activation
+ *   H     one of 256, 384, 512, 640, 768, 1024 (the sizes whose rows a wave keeps in registers);
+ *         any other H: CWR_ERR_SHAPE, and the caller runs cwr_join + cwr_joint_forward instead
+ *   h_out (R, H) or NULL: receives the joint rows, bit-identical to cwr_join's, for a backward pass
+ *         that needs them (cwr_joint_backward, the weight-gradient product, cwr_join_backward)
+ * A cell that lies outside f or g (lx[n] > T_pad or ly[n]+1 > Up_pad) raises CWR_FLAG_BAD_LENGTH
+ * and counts as a row of zeros, as in cwr_join.  Everything else as for cwr_joint_forward. */
+int cwr_joint_forward_fg(const void* f, const void* g, int act, int64_t T_pad, int64_t Up_pad, void* h_out,
+                         const void* w, const float* bias, int dtype, int64_t R, int64_t H, int64_t V,
+                         const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
+                         int64_t N, int32_t blank, int64_t max_u, void* workspace, size_t workspace_bytes,
+                         int64_t* row_off, int64_t* lab_off, int32_t* status, int32_t* rowinfo, float* lse,
+                         float* grads, float* costs, void* stream);
+
 /* Backward of cwr_joint_forward, one block of rows at a time: the logits of rows [0, R) of the block
  * are formed again on the matrix cores (fp32 accumulators) and turned in registers into
  *   dlogits[r, v] = g * (softmax(logits_r)[v] * gamma_r + grads[r,0] [v == blank] + grads[r,1] [v == label]),

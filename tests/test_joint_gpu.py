@@ -368,3 +368,131 @@ def test_joiner_module_loss_agrees_with_the_stored_logits_route():
         assert torch.isfinite(a).all()
         cos = torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0)
         assert float(cos) > 0.99, float(cos)
+
+
+# ----------------------------------------------------------------------------- the joiner's whole chain in one kernel
+def make_fg(lx, ly, H, seed, dtype, T_extra=2, U_extra=1):
+    rng = np.random.default_rng(seed)
+    N = len(lx)
+    T, Up = int(max(lx)) + T_extra, int(max(ly)) + 1 + U_extra  # padded beyond the longest sequence
+    f = torch.from_numpy(rng.standard_normal((N, T, H)).astype(np.float32)).to(TDT[dtype])
+    g = torch.from_numpy(rng.standard_normal((N, Up, H)).astype(np.float32)).to(TDT[dtype])
+    return f, g
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("act", [None, "tanh", "relu"])
+@pytest.mark.parametrize("lx,ly,H,V", [([9, 5, 12, 1], [3, 0, 7, 4], 256, 128), ([40, 33, 17], [12, 20, 5], 512, 300),
+                                       ([25, 31], [20, 9], 768, 257), ([14, 6], [5, 130], 384, 64)])
+def test_joiner_chain_forward_matches_oracle(dtype, act, lx, ly, H, V):
+    """cwr_joint_forward_fg: rows act(f[n,t] + g[n,u]) formed in the kernel.  Oracle: join_rows in
+    float64, rounded once to the 16-bit type (the kernel's one rounding), joint_logits, fused-mode
+    loss.  The rows the kernel leaves behind on request are bit-identical to compact_join's, and the
+    results do not depend on whether it leaves them."""
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd.joiner import _ACTS
+    j = make_joint(lx, ly, H, V, seed=21, dtype=dtype, scale=3.0)
+    f, g = make_fg(lx, ly, H, 22, dtype)
+    h64 = orc.join_rows(f.double().numpy(), g.double().numpy(), j["lx"], j["ly"], act)
+    h16 = torch.from_numpy(h64).to(TDT[dtype])
+    z = orc.joint_logits(h16.double().numpy(), j["w"].double().numpy(), j["b"].numpy())
+    ref = orc.loss_and_grad(z, j["lx"], j["yp"], j["ly"], 0, "fused", want_dense=False)
+    lxd, lyd = torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV)
+    yd = torch.from_numpy(j["yp"]).to(DEV)
+    fd, gd, wd, bd = f.to(DEV), g.to(DEV), j["w"].to(DEV), j["b"].to(DEV)
+    outs = []
+    for keep in (False, True):
+        costs, st, h = pkg.loss.joint_forward_fg(fd, gd, _ACTS[act], wd, bd, lxd, yd, lyd, 0, j["R"], keep_rows=keep)
+        torch.cuda.synchronize()
+        assert int(st.status[0].item()) == 0
+        # a row's rounding to 16 bits may differ from the oracle's by one ulp of the type where the
+        # float32 sum sits on a rounding boundary: the tolerances of the stored-rows route apply
+        np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=2e-4 if dtype == "bf16" else 3e-5)
+        outs.append((costs.cpu().numpy(), st.lse.cpu().numpy(), st.grads.cpu().numpy()))
+        if keep:
+            hj = pkg.compact_join(fd, gd, lxd, lyd, act, total_rows=j["R"])
+            assert torch.equal(h, hj)
+            # and from those very rows the stored-rows entry point gives the same bits
+            c2, st2 = pkg.joint_forward(hj, wd, bd, lxd, yd, lyd, 0)
+            assert torch.equal(c2, costs) and torch.equal(st2.lse, st.lse) and torch.equal(st2.grads, st.grads)
+            z2 = orc.joint_logits(hj.double().cpu().numpy(), j["w"].double().numpy(), j["b"].numpy())
+            ref2 = orc.loss_and_grad(z2, j["lx"], j["yp"], j["ly"], 0, "fused", want_dense=False)
+            np.testing.assert_allclose(costs.cpu().numpy(), ref2["costs"], rtol=LOSS_RTOL)
+            np.testing.assert_allclose(st.grads.cpu().numpy(), ref2["G"], rtol=0, atol=GRAD_ATOL)
+            np.testing.assert_allclose(st.lse.cpu().numpy(), ref2["lse"], rtol=2e-6, atol=2e-5)
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a, b)
+
+
+def test_joiner_chain_flags_cells_outside_its_inputs_and_refuses_other_joint_sizes():
+    import compactwarprnntloss_amd as pkg
+    from compactwarprnntloss_amd import _lib
+    j = make_joint([6, 4], [3, 2], 256, 64, seed=5, dtype="bf16")
+    f, g = make_fg([6, 4], [3, 2], 256, 6, "bf16", T_extra=-1, U_extra=0)  # one frame short of the longest sequence
+    lxd, lyd = torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV)
+    yd = torch.from_numpy(j["yp"]).to(DEV)
+    costs, st, _ = pkg.loss.joint_forward_fg(f.to(DEV), g.to(DEV), 1, j["w"].to(DEV), None, lxd, yd, lyd, 0, j["R"])
+    torch.cuda.synchronize()
+    assert int(st.status[0].item()) & _lib.FLAG_BAD_LENGTH
+    assert torch.isfinite(costs).all()
+    f2, g2 = make_fg([6, 4], [3, 2], 96, 7, "bf16")
+    with pytest.raises(RuntimeError):
+        pkg.loss.joint_forward_fg(f2.to(DEV), g2.to(DEV), 1, j["w"][:, :96].contiguous().to(DEV), None, lxd, yd, lyd, 0, j["R"])
+    lib = _lib.load()
+    A = 1 << 20
+    assert lib.cwr_joint_forward_fg(A, A, 1, 8, 5, None, A, None, _lib.BF16, 100, 96, 64, A, A, A, 3, 6, 2, 0, 3, A,
+                                    1 << 20, A, A, A, A, A, A, A, None) == 4      # CWR_ERR_SHAPE: not a resident size
+    assert lib.cwr_joint_forward_fg(A, A, 7, 8, 5, None, A, None, _lib.BF16, 100, 256, 64, A, A, A, 3, 6, 2, 0, 3, A,
+                                    1 << 20, A, A, A, A, A, A, A, None) == 3      # CWR_ERR_MODE: activation
+    assert lib.cwr_joint_forward_fg(None, A, 1, 8, 5, None, A, None, _lib.BF16, 100, 256, 64, A, A, A, 3, 6, 2, 0, 3,
+                                    A, 1 << 20, A, A, A, A, A, A, A, None) == 1   # CWR_ERR_NULL
+
+
+@pytest.mark.parametrize("act", [None, "tanh", "relu"])
+@pytest.mark.parametrize("reduction", ["mean", "none"])
+def test_fused_joiner_loss_gradients(act, reduction):
+    """fused_joiner_loss -> (df, dg, dW, dbias): identical to compact_join + fused_joint_loss (the same
+    kernels behind both, the rows bit-identical), and within the 16-bit tolerances of the oracle's
+    chain rule (dense fused gradient of the float64 logits, joint_backward, join_rows_backward)."""
+    import compactwarprnntloss_amd as pkg
+    lx, ly, H, V = [40, 33, 17], [12, 20, 5], 256, 300
+    j = make_joint(lx, ly, H, V, seed=31, dtype="bf16", scale=3.0)
+    f, g = make_fg(lx, ly, H, 32, "bf16")
+    N = j["N"]
+    w8 = np.random.default_rng(2).uniform(0.5, 1.5, N)
+    go = np.full(N, 1.0 / N) if reduction == "mean" else w8
+    lxd, lyd = torch.from_numpy(j["lx"]).to(DEV), torch.from_numpy(j["ly"]).to(DEV)
+    yd = torch.from_numpy(j["yp"]).to(DEV)
+    wt = torch.from_numpy(w8).to(DEV).float()
+
+    def run(chain):
+        fd, gd = f.to(DEV).requires_grad_(True), g.to(DEV).requires_grad_(True)
+        W, b = j["w"].to(DEV).requires_grad_(True), j["b"].to(DEV).requires_grad_(True)
+        red = "mean" if reduction == "mean" else "none"
+        if chain:
+            out = pkg.fused_joiner_loss(fd, gd, W, b, lxd, yd, lyd, 0, red, act, total_rows=j["R"], chunk_rows=257,
+                                        one_kernel=True)
+        else:
+            h = pkg.compact_join(fd, gd, lxd, lyd, act, total_rows=j["R"])
+            out = pkg.fused_joint_loss(h, W, b, lxd, yd, lyd, 0, red, chunk_rows=257)
+        loss = out if reduction == "mean" else (out * wt).sum()
+        loss.backward()
+        torch.cuda.synchronize()
+        return [t.grad for t in (fd, gd, W, b)], loss.detach()
+
+    got, loss = run(True)
+    two, loss2 = run(False)
+    assert torch.equal(loss, loss2)
+    for a, b_, name in zip(got, two, ("df", "dg", "dW", "dbias")):
+        assert torch.equal(a, b_), name
+    # oracle
+    f64, g64 = f.double().numpy(), g.double().numpy()
+    h16 = pkg.compact_join(f.to(DEV), g.to(DEV), lxd, lyd, act, total_rows=j["R"]).double().cpu().numpy()
+    z = orc.joint_logits(h16, j["w"].double().numpy(), j["b"].numpy())
+    ref = orc.loss_and_grad(z, j["lx"], j["yp"], j["ly"], 0, "fused", grad_out=go, want_dense=True)
+    dh_ref, dw_ref, db_ref = orc.joint_backward(ref["grad"], h16, j["w"].double().numpy())
+    df_ref, dg_ref = orc.join_rows_backward(dh_ref, f64, g64, j["lx"], j["ly"], act)
+    for a, want, name in zip(got, (df_ref, dg_ref, dw_ref, db_ref), ("df", "dg", "dW", "dbias")):
+        a = a.double().cpu().numpy()
+        scale = np.abs(want).max()
+        np.testing.assert_allclose(a, want, rtol=2e-2, atol=2e-2 * scale, err_msg=name)
