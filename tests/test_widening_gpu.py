@@ -38,8 +38,9 @@ def _lp_of(b, n, fused):
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("lx,ly,sigma", [
     ([9, 5, 12, 1], [3, 0, 7, 4], 1.0),          # small, ragged, U=0 and T=1
-    ([40, 150], [70, 130], 1.0),                 # two and three strips of 64 labels
-    ([30, 7], [20, 600], 1.0),                   # ten strips: the sequential log-domain walk
+    ([40, 150], [70, 130], 1.0),                 # one and two strips of 128 labels
+    ([30, 7, 20], [20, 600, 300], 1.0),          # five and three strips, walked concurrently
+    ([6, 9], [1100, 40], 1.0),                   # nine strips: the sequential log-domain walk
     ([60, 33], [25, 64], 40.0),                  # steep logits: the per-sequence log-domain walk
 ])
 def test_alpha_beta_export_matches_oracle(fused, lx, ly, sigma):
