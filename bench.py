@@ -108,6 +108,9 @@ def main():
                     help="also time the compact joiner front (broadcast sum + tanh for valid cells, H=512, in the "
                          "batch's storage type) and its backward at the same lengths (reported under 'joiner_op'; "
                          "not part of 'value')")
+    ap.add_argument("--with-long-labels", action="store_true",
+                    help="also time the forward call and its lattice stage on N=4, T=1250 and U = 300 ... 1200 labels "
+                         "(log-prob mode, V=4: the lattice dominates; reported under 'long_labels')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so that a counter run can scale "
                          "FETCH_SIZE / WRITE_SIZE against it")
@@ -253,6 +256,39 @@ def main():
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": traffic, "traffic_source": traffic_source},
     }
+
+    if args.with_long_labels:
+        # Label sequences beyond one workgroup's concurrent strips: up to 1023 labels a sequence is walked
+        # by one wave per strip of 128 labels at once; from 1024 on one wave walks the strips in turn.
+        import ctypes as C
+        lib = pkg._lib.load()
+        rows = []
+        for U in (300, 511, 600, 1000, 1023, 1200):
+            Nl, Tl, Vl = 4, 1250, 4
+            lxl = torch.full((Nl,), Tl, dtype=torch.int32, device=dev)
+            lyl = torch.full((Nl,), U, dtype=torch.int32, device=dev)
+            Rl = Nl * Tl * (U + 1)
+            xl = torch.log_softmax(torch.randn((Rl, Vl), device=dev), dim=1)
+            yl = torch.randint(1, Vl, (Nl, U), dtype=torch.int32, device=dev)
+            cl, stl = pkg.rnnt_forward(xl, lxl, yl, lyl, 0, False)
+            stage = (C.c_float * 4)()
+            runs = []
+            for _ in range(7):
+                rc = lib.cwr_debug_forward_stage_times(
+                    xl.data_ptr(), pkg.loss._DTYPES[xl.dtype], Rl, Vl, lxl.data_ptr(), lyl.data_ptr(), yl.data_ptr(), U,
+                    yl.numel(), Nl, 0, pkg._lib.MODE_LOGPROB, stl.max_u, stl.workspace.data_ptr(),
+                    stl.workspace.numel(), stl.row_off.data_ptr(), stl.lab_off.data_ptr(), stl.status.data_ptr(),
+                    stl.rowinfo.data_ptr(), None, stl.grads.data_ptr(), cl.data_ptr(),
+                    torch.cuda.current_stream().cuda_stream, stage)
+                if rc != 0:
+                    sys.exit("cwr_debug_forward_stage_times: " + pkg._lib.strerror(rc))
+                runs.append(list(stage))
+            med = [sorted(r[i] for r in runs)[len(runs) // 2] for i in range(4)]
+            rows.append({"U": U, "strips_of_128": (U + 128) // 128, "lattice_us": round(med[2], 1),
+                         "forward_call_us": round(sum(med), 1),
+                         "lattice_ns_per_diagonal": round(med[2] * 1e3 / (Tl + U), 1)})
+            del xl, yl, cl, stl
+        result["long_labels"] = {"N": 4, "T": 1250, "V": 4, "mode": "log-prob", "cases": rows}
 
     if args.with_pack:
         Tm, Up = int(cfg["lx"].max()), int(cfg["ly"].max()) + 1
