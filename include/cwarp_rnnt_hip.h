@@ -71,7 +71,8 @@ enum cwr_flag {
                                    more than 1e-5, so that a likelihood within rounding of 1 does
                                    not count) for some sequence; the cost is their mean, as in the
                                    reference (cwarp_cuda_rnnt_kernel.cu:356-364, which prints) */
-    CWR_FLAG_U_TOO_LARGE = 16,  /* some ly exceeds the max_u given to the call */
+    CWR_FLAG_U_TOO_LARGE = 16,  /* some ly exceeds the max_u given to the call, or some lx exceeds
+                                   2^19 frames */
     CWR_FLAG_INTERNAL = 32      /* a bounded wait inside a kernel ran out (the cost of the sequence it
                                    happened in is NaN) */
 };
@@ -127,7 +128,8 @@ int cwr_offsets(const int32_t* lx, const int32_t* ly, int64_t N, int64_t R,
  *   x        (R,V) of `dtype`, contiguous
  *   lx, ly   (N,) int32 frame / label counts;  y, y_stride: labels (see above)
  *   max_u    an upper bound of max(ly) known to the host (e.g. the padded label width); a
- *            sequence with more labels is skipped (cost NaN, CWR_FLAG_U_TOO_LARGE)
+ *            sequence with more labels, or with more than 2^19 frames, is skipped (cost NaN,
+ *            CWR_FLAG_U_TOO_LARGE)
  * outputs
  *   row_off, lab_off (N+1) int64;  status 4 x int32 (word 0: CWR_FLAG_* bits; the others are
  *            scratch of the call)
