@@ -222,6 +222,8 @@ def main():
         lat_runs.append(list(stage))
     lat = [sorted(r[i] for r in lat_runs)[len(lat_runs) // 2] for i in range(4)]  # medians
     diagonals = int((cfg["lx"].astype(np.int64) + cfg["ly"]).max())
+    # the walk serves two label positions per lane and step: T + ceil((U+1)/2) - 1 steps per sequence
+    walk_steps = int((cfg["lx"].astype(np.int64) + (cfg["ly"].astype(np.int64) + 2) // 2 - 1).max())
 
     grad_bytes = R * V * 2 * esize
     achieved = grad_bytes / (bwd_ms * 1e-3) / 1e9
@@ -250,6 +252,8 @@ def main():
                        "fill": round(lat[3], 2), "grad": round(bwd_ms * 1e3, 2),
                        "lattice_ns_per_diagonal": round(lat[2] * 1e3 / diagonals, 1),
                        "diagonals_longest_sequence": diagonals,
+                       "lattice_ns_per_walk_step": round(lat[2] * 1e3 / walk_steps, 1),
+                       "walk_steps_longest_sequence": walk_steps,
                        "how": "medians of HIP-event intervals between the stages of one forward call "
                               "(cwr_debug_forward_stage_times); grad = the backward call"},
         "roofline": {"bound": "hbm", "kernel": "k_grad (cwr_backward)", "achieved": round(achieved, 1),

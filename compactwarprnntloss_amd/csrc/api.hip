@@ -49,14 +49,16 @@ struct Layout {
 // Upper bounds, from what the host knows (N, R, max_u), of the lattice slots and boundary-stream
 // entries a batch can need: every strip adds at most (63 + 2*kRowShift) * 128 padding slots to the
 // R real cells (one padding row per lane but the first, and the rows in front and behind), a
-// sequence one slot to keep its size even, and a sequence has at most ceil((max_u+1)/128) strips.
+// sequence's last strip one column of padding when its width is odd (one slot per frame: R of them
+// for a batch without labels, none when every width is even), and a sequence has at most
+// ceil((max_u+1)/128) strips.
 static Layout layout_for(i64 N, i64 R, i64 max_u) {
     Layout l;
     const i64 n = N > 0 ? N : 0, r = R > 0 ? R : 0, mu = max_u > 0 ? max_u : 0;
     const i64 strips = strip_count(mu + 1);
-    i64 by_strips = r + n * (strips * (63 + 2 * kRowShift) * kStripCols + 1);
-    // each cell is also at most 63 + 2*kRowShift slots of padding away (a strip of one frame)
-    i64 by_rows = r * (64 + 2 * kRowShift) + n;
+    i64 by_strips = 2 * r + n * strips * (63 + 2 * kRowShift) * kStripCols;
+    // a strip holds at most 2 * (1 + 2*kRowShift) slots per cell (one frame, one column)
+    i64 by_rows = r * (2 + 4 * kRowShift);
     l.slot_cap = by_strips < by_rows ? by_strips : by_rows;
     if (l.slot_cap < 0) l.slot_cap = 0;
     // boundary streams: (S-1)*(T+kBndPad) per sequence, with (S-1)*128 <= U < rows of the sequence

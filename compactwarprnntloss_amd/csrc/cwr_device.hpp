@@ -169,9 +169,11 @@ template <typename T, int VEC> struct alignas(sizeof(T) * VEC) PackT { T e[VEC];
 // of kStripCols = 128 label positions; strip s holds nl = min(128, U+1-128s) columns, two per lane
 // of the wave that walks it (lane j: columns 2j and 2j+1 of the strip).  Inside a strip, cell
 // (t, u = 128s+c) is stored at row t + c/2 + kRowShift, column c, of a dense
-// (T + ceil(nl/2) - 1 + 2*kRowShift) x nl array: a wave that walks the strip with lane j one frame
-// behind lane j-1 touches one contiguous row per step, at a constant pitch.  The rows above and
-// below, and the two triangles of slots that hold no cell, are padding.
+// (T + ceil(nl/2) - 1 + 2*kRowShift) x pitch array, pitch = nl rounded up to even: a wave that
+// walks the strip with lane j one frame behind lane j-1 touches one contiguous row per step, at a
+// constant pitch, and every lane's pair of columns is one aligned 16-byte access (a strip of odd
+// width has a column of padding for its last lane's second column).  The rows above and below, and
+// the two triangles of slots that hold no cell, are padding too.
 constexpr int kPF = 16;               // prefetch depth of the lattice walk, in rows
 constexpr int kRowShift = 2 * kPF;    // padding rows in front of (and behind) a strip
 constexpr int kBndPad = 192;          // entries a boundary stream holds beyond T
@@ -179,18 +181,19 @@ constexpr int kStripCols = 128;       // label positions per strip
 constexpr int kStripShift = 7;        // log2(kStripCols)
 
 __host__ __device__ __forceinline__ i64 strip_lanes(i64 nl) { return (nl + 1) >> 1; }
+__host__ __device__ __forceinline__ i64 strip_pitch(i64 nl) { return (nl + 1) & ~(i64)1; }
 __host__ __device__ __forceinline__ i64 strip_rows(i64 T, i64 nl) { return T + strip_lanes(nl) - 1 + 2 * kRowShift; }
 __host__ __device__ __forceinline__ i64 strip_count(i64 Up) { return (Up + kStripCols - 1) >> kStripShift; }
 __host__ __device__ __forceinline__ i64 lattice_slots(i64 T, i64 Up) {
     i64 full = (Up - 1) >> kStripShift;  // strips before the last one are full
     i64 nl = Up - (full << kStripShift);
-    // an even number of slots: every strip then starts on a 16-byte boundary of the fp64 arrays
-    return (full * strip_rows(T, kStripCols) * kStripCols + strip_rows(T, nl) * nl + 1) & ~(i64)1;
+    // always an even number of slots: every strip starts on a 16-byte boundary of the fp64 arrays
+    return full * strip_rows(T, kStripCols) * kStripCols + strip_rows(T, nl) * strip_pitch(nl);
 }
 __host__ __device__ __forceinline__ i64 lattice_slot(i64 t, i64 u, i64 T, i64 Up) {
     i64 s = u >> kStripShift, c = u & (kStripCols - 1);
     i64 nl = Up - (s << kStripShift) < kStripCols ? Up - (s << kStripShift) : kStripCols;
-    return s * strip_rows(T, kStripCols) * kStripCols + (t + (c >> 1) + kRowShift) * nl + c;
+    return s * strip_rows(T, kStripCols) * kStripCols + (t + (c >> 1) + kRowShift) * strip_pitch(nl) + c;
 }
 __host__ __device__ __forceinline__ i64 boundary_entries(i64 T, i64 Up) {
     return ((Up - 1) >> kStripShift) * (T + kBndPad);

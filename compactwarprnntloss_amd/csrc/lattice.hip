@@ -70,7 +70,7 @@ __device__ __forceinline__ void buf_store_i32(__amdgpu_buffer_rsrc_t r, int voff
 // values -> their scales) overlap across waves.
 constexpr int kFillSlots = 256;
 __host__ __device__ __forceinline__ i64 strip_chunks(i64 T, i64 nl) {
-    return ((T + strip_lanes(nl) - 1) * nl + kFillSlots - 1) / kFillSlots;
+    return ((T + strip_lanes(nl) - 1) * strip_pitch(nl) + kFillSlots - 1) / kFillSlots;
 }
 __host__ __device__ __forceinline__ i64 fill_chunks(i64 T, i64 Up) {
     const i64 full = (Up - 1) >> kStripShift;
@@ -303,14 +303,8 @@ __device__ __forceinline__ LaneCols lane_cols(int lane, int nl, int bytes) {
     return lc;
 }
 
-// The records of a lane's two columns in one row: one 16-byte load, or two 8-byte loads when the
-// strip's last lane has one column only (the missing one then reads as zeros).
-template <bool ODD>
+// The records of a lane's two columns in one row, as one 16-byte load.
 __device__ __forceinline__ float4 load_pair(__amdgpu_buffer_rsrc_t r, const LaneCols v, int soff) {
-    if (ODD) {
-        const float2 a = buf_load_f2(r, v.c0, soff), b = buf_load_f2(r, v.c1, soff);
-        return make_float4(a.x, a.y, b.x, b.y);
-    }
     const v4i x = __builtin_amdgcn_raw_buffer_load_b128(r, v.c0, soff, 0);
     return make_float4(__int_as_float(x.x), __int_as_float(x.y), __int_as_float(x.z), __int_as_float(x.w));
 }
@@ -320,7 +314,7 @@ __device__ __forceinline__ float4 load_pair(__amdgpu_buffer_rsrc_t r, const Lane
 // lane that holds "no path" there (junk in those records could be a NaN, which nothing survives).
 template <bool BETA>
 __device__ __forceinline__ void clear_leading(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
-    const int p8 = nl * 8;
+    const int p8 = (int)strip_pitch(nl) * 8;
     const int nlane = (int)strip_lanes(nl);
     const LaneCols vc = lane_cols(lane, nl, 8);
 #pragma unroll 4
@@ -339,10 +333,16 @@ __device__ __forceinline__ void clear_leading(__amdgpu_buffer_rsrc_t r_cell, int
 // Both directions of a sequence clear the same records; nothing else is ever written to them.
 template <bool BETA>
 __device__ __forceinline__ void clear_around(__amdgpu_buffer_rsrc_t r_cell, int T, int nl, int lane) {
-    const int p8 = nl * 8;
+    const int p8 = (int)strip_pitch(nl) * 8;
     const int nlane = (int)strip_lanes(nl);
     const int Q = T + nlane - 1;
     const LaneCols vc = lane_cols(lane, nl, 8);
+    // a strip of odd width: the column of padding that completes its last lane's pair, in every row
+    // (the lanes share the rows out; a few stores each)
+    if (nl & 1) {
+        const int rows = (int)strip_rows(T, nl);
+        for (int row = lane; row < rows; row += 64) buf_store_zero8(r_cell, row * p8 + nl * 8, 0);
+    }
     // row j of the cells' bounding box: lanes > j have not started; in row T+j lanes <= j have
     // finished; one store covers both (the per-lane offset picks the row)
 #pragma unroll 4
@@ -377,19 +377,53 @@ constexpr unsigned kLowHigh = (unsigned)(1023 + kLowExp) << 20;    // high word 
 constexpr unsigned kHighHigh = (unsigned)(1023 + kHighExp) << 20;  // high word of 2^kHighExp
 
 // ---- scaled linear-domain walk (strips concurrent, LDS rings) -------------------------------
+// The value entering the strip at step J of a block, moved into the edge lane's copy of `nbr`.  Lane
+// J of every row of 16 lanes holds step J's entry; the edge lane (lane 0 for alpha, lane 63 for
+// beta) reads it with a shift inside its row.  Under the row / bank masks the move writes the four
+// lanes at the edge lane's end of the wave at most, and the shift of `pass` from the neighbouring
+// lane, which follows, overwrites every lane but the edge lane.  Two moves per step, against two
+// v_readlane and a multiply-add.
+template <bool BETA, int J>
+__device__ __forceinline__ double place_entry(double nbr, double e) {
+    constexpr int ctrl = BETA ? (J == kPF - 1 ? 0xE4 : DPP_ROW_SHR + (kPF - 1 - J)) : (J == 0 ? 0xE4 : DPP_ROW_SHL + J);
+    return dpp_f64<ctrl, BETA ? 0x8 : 0x1, BETA ? 0x8 : 0x1>(nbr, e);
+}
+template <bool BETA>
+__device__ __forceinline__ double place_entry(double nbr, double e, int j) {
+    static_assert(kPF == 16, "one case per step of a block");
+    switch (j) {
+        case 0: return place_entry<BETA, 0>(nbr, e);
+        case 1: return place_entry<BETA, 1>(nbr, e);
+        case 2: return place_entry<BETA, 2>(nbr, e);
+        case 3: return place_entry<BETA, 3>(nbr, e);
+        case 4: return place_entry<BETA, 4>(nbr, e);
+        case 5: return place_entry<BETA, 5>(nbr, e);
+        case 6: return place_entry<BETA, 6>(nbr, e);
+        case 7: return place_entry<BETA, 7>(nbr, e);
+        case 8: return place_entry<BETA, 8>(nbr, e);
+        case 9: return place_entry<BETA, 9>(nbr, e);
+        case 10: return place_entry<BETA, 10>(nbr, e);
+        case 11: return place_entry<BETA, 11>(nbr, e);
+        case 12: return place_entry<BETA, 12>(nbr, e);
+        case 13: return place_entry<BETA, 13>(nbr, e);
+        case 14: return place_entry<BETA, 14>(nbr, e);
+        default: return place_entry<BETA, 15>(nbr, e);
+    }
+}
+
 // Every LANE carries its own scale: the values of its two columns are probabilities times 2^C, with
 // C renewed at the start of every block of kPF steps so that the largest of the lane's own values
 // and of what its neighbour is about to hand over sits at 2^kLinTarget.  A value arriving from the
-// neighbouring lane is brought to the lane's scale by one v_ldexp_f64 with the (block-constant)
-// difference of the two scales.  Like a logarithm, this loses nothing across lanes, however far
+// neighbouring lane is brought to the lane's scale by the (block-constant) power of two that
+// separates the two scales, inside the multiply-add that takes it in.  Like a logarithm, this loses nothing across lanes, however far
 // apart their magnitudes are: the only thing that can underflow is a summand that is negligible
 // next to the other summand of the SAME cell, or one of a lane's two columns next to the other.
 // Within a block a lane's value can still drift out of the fp64 range (a run of extreme factors,
 // or a much larger magnitude arriving from several columns away), which the range check catches.
-// ODD: the strip's last lane has one column only (nl odd); the pair is then stored as two 8-byte
-// values, the missing one at the rejected offset.  seed_col: column of this strip that holds the
-// start cell of the walk, or -1.  Returns false when the check failed.
-template <bool BETA, bool HAS_IN, bool HAS_OUT, bool ODD>
+// In a strip of odd width the last lane's second column is the layout's column of padding: zero
+// probabilities in, zeros out.  seed_col: column of this strip that holds the start cell of the
+// walk, or -1.  Returns false when the check failed.
+template <bool BETA, bool HAS_IN, bool HAS_OUT>
 __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const int seed_col, const int in_shift,
                                                 const int out_shift, const float2* lp_strip,
                                                 double* out_strip, int* scale_strip, const Ring rin,
@@ -399,11 +433,11 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     const int Q = T + nlane - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    const int p8 = nl * 8, p4 = nlane * 4;
+    const int pitch = (int)strip_pitch(nl);
+    const int p8 = pitch * 8, p4 = nlane * 4;
     const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p8);
-    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_sc = make_rsrc(scale_strip, (i64)nblocks * p4);
-    const LaneCols vo = lane_cols(lane, nl, 8);  // a lane's two columns in a row of 8-byte records
+    const LaneCols vo = lane_cols(lane, pitch, 8);  // a lane's two columns in a row of 8-byte records
     const LaneCols vp = vo;
     const int vo_sc = lane < nlane ? lane * 4 : kOob;
     constexpr int in_lane = BETA ? 63 : 0;  // a strip that takes values in is 128 wide
@@ -414,21 +448,21 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     clear_around<BETA>(r_cell, T, nl, lane);
 
     const int row0 = (BETA ? Q - 1 : 0) + kRowShift;  // row of step 0
-    int qi = row0;                                    // row of the current step
-    int mi = BETA ? row0 - 1 : row0;                  // row that holds the current step's multipliers
+    const int mi = BETA ? row0 - 1 : row0;            // row that holds step 0's multipliers
     float4 ring[kPF];  // (blank, label) probabilities of the two columns, rows mi .. mi+dq*(kPF-1)
 #pragma unroll
-    for (int j = 0; j < kPF; ++j) ring[j] = load_pair<ODD>(r_cell, vp, (mi + dq * j) * p8);
+    for (int j = 0; j < kPF; ++j) ring[j] = load_pair(r_cell, vp, (mi + dq * j) * p8);
     int C = kLinTarget;  // this lane's scale exponent
     int d = 0;           // C minus the scale exponent of the lane the neighbour values come from
     // alpha[0][0] = 1; beta[T-1][U] = blank probability of that cell
     double own0 = 0.0, own1 = 0.0;
-    float l_row0 = 0.f;  // beta: L(t,c0) of the row of step 0
+    float l_row0 = 0.f, l_row1 = 0.f;  // beta: L(t,c0), L(t,c1) of the row of step 0
     {
         const bool seed0 = seed_col == 2 * lane, seed1 = seed_col == 2 * lane + 1;
         if (BETA) {
             const float pb = buf_load_f(r_cell, (seed0 || seed1) ? seed_col * 8 : kOob, row0 * p8);
             l_row0 = buf_load_f(r_cell, vp.c0 == kOob ? kOob : vp.c0 + 4, row0 * p8);
+            l_row1 = buf_load_f(r_cell, vp.c1 == kOob ? kOob : vp.c1 + 4, row0 * p8);
             const double sv = __builtin_ldexp((double)pb, kLinTarget);
             own0 = seed0 ? sv : 0.0;
             own1 = seed1 ? sv : 0.0;
@@ -438,25 +472,40 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
     }
     double pass = 0.0;
     double nbr = 0.0;  // the edge lane has no neighbour: it keeps "no path" here for good
-    // alpha applies its own cells' probabilities: (B0, L0, B1, L1) of the row.  beta applies
-    // B(t-1,c0), B(t-1,c1) of the row before, L(t,c0) of the row itself (kept from the step before)
-    // and L(t,c0-1), which is the second label probability the lane on its left holds for the row
-    // before (lane 0 gets 0: nobody reads its `pass`)
+    // alpha applies its own cells' probabilities: (B0, L0, B1, L1) of the row, and hands on
+    // alpha(t,c1) * L1.  beta applies B(t-1,c0), B(t-1,c1) of the row before and L(t,c0), L(t,c1) of
+    // the row itself (kept from the step before); it hands on plain beta(t,c0), and the lane that
+    // takes it in applies its own L(t,c1) together with the change of scale, whether the value comes
+    // from the lane on its right or, for the edge lane, from the strip on the right.
     double mB0 = (double)ring[0].x, mB1 = (double)ring[0].z;
     double mL0 = BETA ? (double)l_row0 : (double)ring[0].y;
-    double mL1 = (double)(BETA ? dpp_f32_or_zero<DPP_WAVE_SHR1>(ring[0].w) : ring[0].w);
+    double mL1 = BETA ? (double)l_row1 : (double)ring[0].w;
     double mL0_next = BETA ? (double)ring[0].y : 0.0;  // beta: L(t-1,c0), for the step after this one
-    const double in_mask = lane == in_lane ? 1.0 : 0.0;
+    double mL1_next = BETA ? (double)ring[0].w : 0.0;  // beta: L(t-1,c1)
+    double pdL = 0.0;                                  // beta: 2^d * L(t,c1)
     unsigned lo_seen = 0xffffffffu, hi_seen = 0u;  // extremes of the cell values' high words (zero excluded)
-    // beta hands on plain beta(t,u+1); the receiving edge column applies its own L(t,u), fetched
-    // one block ahead by the lanes that prepare the incoming entries
+    // lane j of every row of 16 prepares the value that enters at step j of a block
     const int jl = lane & (kPF - 1);
-    constexpr int edge_off = (kStripCols - 1) * 8 + 4;
-    float edge = 0.f;
-    if (BETA && HAS_IN) edge = buf_load_f(r_cell, max(row0 - jl, 0) * p8 + edge_off, 0);
+    // Row addressing of the step loop.  A lone wave pays five to eight clocks for EVERY instruction
+    // it issues, scalar ones included, so the rows of a block are reached without any arithmetic per
+    // step: the kPF row offsets inside a block never change and sit in scalar registers, and the
+    // block's position goes into the base address of the two descriptors, once per block.
+    int srow[kPF];
+#pragma unroll
+    for (int j = 0; j < kPF; ++j) {
+        srow[j] = (BETA ? kPF - 1 - j : j) * p8;
+        asm volatile("" : "+s"(srow[j]));  // a value of its own: never re-derived inside the loop
+    }
+    const i64 blk_bytes = (i64)dq * kPF * p8;
+    // lowest row a block's loads (kPF rows ahead of its steps) and stores touch; never below row 0
+    const char* cell_blk = reinterpret_cast<const char*>(lp_strip) + (i64)(BETA ? mi - 2 * kPF + 1 : mi + kPF) * p8;
+    char* out_blk = reinterpret_cast<char*>(out_strip) + (i64)(BETA ? row0 - kPF + 1 : row0) * p8;
     settle_loads();
     int k0 = 0;
-    for (int blk = 0; blk < nblocks; ++blk, k0 += kPF) {
+    for (int blk = 0; blk < nblocks; ++blk, k0 += kPF, cell_blk += blk_bytes, out_blk += blk_bytes) {
+        // sixteen rows from the block's base, of the rows * p8 bytes the strip has from ITS base
+        const __amdgpu_buffer_rsrc_t r_cell_b = make_rsrc(cell_blk, rows * p8);
+        const __amdgpu_buffer_rsrc_t r_out_b = make_rsrc(out_blk, rows * p8);
         // The two counters and (speculatively) the incoming entries in ONE LDS round trip: LDS
         // serves a wave's requests in order, so entries read after a counter that already shows them
         // produced are the produced ones.  Only a counter that falls short sends the wave polling.
@@ -491,11 +540,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         double e_lane = 0.0;  // lane j < kPF: the value entering at step k0+j
         int cp = 0;           // ... and the scale it was produced at
         if (HAS_IN) {
-            double ev = en_first;
-            if (BETA) {
-                ev *= (double)edge;
-                edge = buf_load_f(r_cell, max(row0 - (k0 + kPF + jl), 0) * p8 + edge_off, 0);
-            }
+            const double ev = en_first;
             // entry k0+j feeds frame k0+j of the edge column: beyond the last frame it is junk
             const bool ok = k0 + jl < T && ev != 0.0;
             cp = cp_first;
@@ -545,26 +590,29 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
         C = Cn;
         d = C - (BETA ? dpp_i32<DPP_WAVE_SHL1>(C, C) : dpp_i32<DPP_WAVE_SHR1>(C, C));
         if (lane >= nlane) d = -8192;  // lanes beyond the strip's width take nothing in: they stay at 0
+        // 2^d as a factor: the neighbour's value then enters through one fused multiply-add instead of
+        // a v_ldexp_f64 and an add.  The product with a power of two is exact, so the sum is the same
+        // but for d below -1022, where the term (2^-1000 of what the lane holds, at most) is dropped
+        // a little earlier.  d above 1023 would overflow whatever it scales, and inf * 0 is a NaN.
+        const double pd = __builtin_ldexp(1.0, min(d, 1023));
+        if (BETA) pdL = pd * mL1;
         if (HAS_IN) e_lane = __builtin_ldexp(e_lane, __builtin_amdgcn_readlane(C, in_lane) - cp);
         buf_store_i32(r_sc, vo_sc, __builtin_amdgcn_readfirstlane(blk * p4), C);  // wave-uniform, and said so
         if (HAS_OUT) rout.scales[(k0 / kPF) & (kRing / kPF - 1)] = __builtin_amdgcn_readlane(C, out_lane);
 #pragma unroll
         for (int j = 0; j < kPF; ++j) {
-            const float4 cn = load_pair<ODD>(r_cell, vp, (mi + dq * kPF) * p8);
+            const float4 cn = load_pair(r_cell_b, vp, srow[j]);
+            if (HAS_IN) nbr = place_entry<BETA>(nbr, e_lane, j);
             nbr = BETA ? dpp_f64<DPP_WAVE_SHL1>(nbr, pass) : dpp_f64<DPP_WAVE_SHR1>(nbr, pass);
             double a0, a1;
             if (BETA) {
-                double o = own1;
-                if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own1);
-                a1 = o + __builtin_ldexp(nbr, d);
+                a1 = __builtin_fma(nbr, pdL, own1);
                 own1 = a1 * mB1;
                 a0 = own0 + a1 * mL0;
                 own0 = a0 * mB0;
-                pass = a0 * mL1;
+                pass = a0;
             } else {
-                double o = own0;
-                if (HAS_IN) o = __builtin_fma(readlane_f64(e_lane, j), in_mask, own0);
-                a0 = o + __builtin_ldexp(nbr, d);
+                a0 = __builtin_fma(nbr, pd, own0);
                 own0 = a0 * mB0;
                 a1 = own1 + a0 * mL0;
                 own1 = a1 * mB1;
@@ -575,12 +623,7 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
                 lo_seen = min(lo_seen, min(h0 - 1u, h1 - 1u));  // zero wraps to the top and drops out
                 if (j % kCheckHigh == 0) hi_seen = max(hi_seen, max(h0, h1));
             }
-            if (ODD) {
-                buf_store_d(r_out, vo.c0, qi * p8, a0);
-                buf_store_d(r_out, vo.c1, qi * p8, a1);
-            } else {
-                buf_store_d2(r_out, vo.c0, qi * p8, a0, a1);
-            }
+            buf_store_d2(r_out_b, vo.c0, srow[j], a0, a1);
             if (HAS_OUT) ring_out[(k0 + j) & (kRing - 1)] = BETA ? a0 : pass;
             const float4 nx = ring[(j + 1) % kPF];
             mB0 = (double)nx.x;
@@ -588,14 +631,14 @@ __device__ __forceinline__ bool sweep_strip_lin(const int T, const int nl, const
             if (BETA) {
                 mL0 = mL0_next;
                 mL0_next = (double)nx.y;
-                mL1 = (double)dpp_f32_or_zero<DPP_WAVE_SHR1>(nx.w);
+                mL1 = mL1_next;
+                mL1_next = (double)nx.w;
+                pdL = pd * mL1;
             } else {
                 mL0 = (double)nx.y;
                 mL1 = (double)nx.w;
             }
             ring[j] = cn;
-            qi += dq;
-            mi += dq;
             // keeps the conversions above inside this step: gathered at the top of the block they
             // would wait for every load in flight
             __builtin_amdgcn_sched_barrier(0);
@@ -641,7 +684,7 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     const int Q = T + nlane - 1;
     const i64 rows = strip_rows(T, nl);
     const int nblocks = (Q + kPF - 1) / kPF;
-    const int p8 = nl * 8;
+    const int p8 = (int)strip_pitch(nl) * 8;
     const __amdgpu_buffer_rsrc_t r_cell = make_rsrc(lp_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_out = make_rsrc(out_strip, rows * p8);
     const __amdgpu_buffer_rsrc_t r_in = make_rsrc(bnd_in, (HAS_IN && !CONC) ? ((i64)T + kBndPad) * 8 : 0);
@@ -772,24 +815,14 @@ __device__ __forceinline__ void sweep_strip_log(const int T, const int nl, const
     if (CONC && HAS_IN) __hip_atomic_store(rin.consumed, 0x7fffffff, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-// A strip's width is odd only when it is the last of its sequence: the alpha walk then has no strip
-// to feed, the beta walk none that feeds it.
 template <bool BETA>
 __device__ __forceinline__ bool lin_dispatch(bool has_in, bool has_out, int T, int nl, int seed_col, int in_shift,
                                              int out_shift, const float2* lp, double* out, int* sc, Ring rin,
                                              Ring rout, const WaitCtl status) {
-    if (nl & 1) {
-        if (BETA) {
-            if (has_out) return sweep_strip_lin<BETA, false, true, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-            return sweep_strip_lin<BETA, false, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-        }
-        if (has_in) return sweep_strip_lin<BETA, true, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-        return sweep_strip_lin<BETA, false, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    }
-    if (has_in && has_out) return sweep_strip_lin<BETA, true, true, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    if (has_in) return sweep_strip_lin<BETA, true, false, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    if (has_out) return sweep_strip_lin<BETA, false, true, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
-    return sweep_strip_lin<BETA, false, false, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_in && has_out) return sweep_strip_lin<BETA, true, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_in) return sweep_strip_lin<BETA, true, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    if (has_out) return sweep_strip_lin<BETA, false, true>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
+    return sweep_strip_lin<BETA, false, false>(T, nl, seed_col, in_shift, out_shift, lp, out, sc, rin, rout, status);
 }
 
 template <bool BETA, bool CONC>
@@ -1082,12 +1115,13 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
             const i64 base = pad + (i64)s * full;
             // first slot of the chunk, counted from the strip's first cell row, as (row, column)
             const unsigned i0 = (local - s * per_full) * (unsigned)kFillSlots;
-            const unsigned q_first = i0 / (unsigned)nl;
-            const int c_first = (int)(i0 - q_first * (unsigned)nl);
-            const float inv_nl = 1.0f / (float)nl;
+            const int pitch = (int)strip_pitch(nl);  // slots per row; one of them padding when nl is odd
+            const unsigned q_first = i0 / (unsigned)pitch;
+            const int c_first = (int)(i0 - q_first * (unsigned)pitch);
+            const float inv_pitch = 1.0f / (float)pitch;
             // the strip after this one, for the cells of this strip's last column
             const int nl2 = (int)s + 1 < S ? ((int)s + 2 == S ? Up - (((int)s + 1) << kStripShift) : kStripCols) : 1;
-            const int lanes2 = (int)strip_lanes(nl2);
+            const int lanes2 = (int)strip_lanes(nl2), pitch2 = (int)strip_pitch(nl2);
             const i64 base2 = base + full;
             LatticeView A, Bv;
             A.v = alpha; A.scale = scale_a; A.pad = pad; A.T = T; A.Up = Up; A.linear = linear_alpha(mode, S); A.beta = false;
@@ -1101,28 +1135,28 @@ __global__ __launch_bounds__(256) void k_fill(const int* __restrict__ lx, const 
             for (int pass = 0; pass < kFillPasses; ++pass) {
                 Raw& w = raw[pass];
                 // slot c_first + 64*pass + lane of the rows from q_first on; at most
-                // nl + kFillSlots < 2^9, so the quotient by nl is exact in fp32
+                // pitch + kFillSlots < 2^9, so the quotient by the pitch is exact in fp32
                 const int il = c_first + pass * 64 + lane;
-                const int dqr = (int)(((float)il + 0.5f) * inv_nl);
+                const int dqr = (int)(((float)il + 0.5f) * inv_pitch);
                 const int q = (int)q_first + dqr;
-                const int col = il - dqr * nl;
+                const int col = il - dqr * pitch;
                 const int l = col >> 1;
                 const int t = q - l;
-                w.ok = q < Q && t >= 0 && t < T;
+                w.ok = q < Q && col < nl && t >= 0 && t < T;
                 const int qs = w.ok ? q : 0, cs = w.ok ? col : 0, ls = w.ok ? l : 0;
                 w.t = qs - ls;
                 w.u = ((int)s << kStripShift) + cs;
-                const i64 slot = base + (i64)(qs + kRowShift) * nl + cs;
+                const i64 slot = base + (i64)(qs + kRowShift) * pitch + cs;
                 // (t+1,u): same column, next strip row, written at step Q-2-q of the beta walk.
                 // (t,u+1): the lane's second column in the same row (step Q-1-q), or the next lane's
                 // first column one row further (step Q-2-q), or column 0 of the next strip in row t.
                 const bool second = (cs & 1) != 0;
                 const bool inside = cs + 1 < nl || !w.ok || (int)s + 1 >= S;
-                const i64 slot_n = inside ? (second ? slot + nl + 1 : slot + 1) : base2 + (i64)(w.t + kRowShift) * nl2;
+                const i64 slot_n = inside ? (second ? slot + pitch + 1 : slot + 1) : base2 + (i64)(w.t + kRowShift) * pitch2;
                 const int kb_d = max(Q - 2 - qs, 0);
                 w.a = alpha[slot];
                 w.cell = lpl[slot];
-                w.bd = beta[slot + nl];
+                w.bd = beta[slot + pitch];
                 w.bn = beta[slot_n];
                 w.ca = w.cbd = w.cbn = 0;
                 if (A.linear) w.ca = scale_a[A.scale_index(base, qs, lanes, ls)];
@@ -1165,7 +1199,7 @@ int launch_fill(const Batch& b, const Workspace& ws, const int* rowinfo, float* 
                 float* reduced) {
     if (b.R == 0) return CWR_OK;
     const i64 strips = strip_count(b.max_u + 1);
-    i64 waves = b.R / kFillSlots + (i64)b.N * strips * (64 * kStripCols / kFillSlots + 1) + 1;
+    i64 waves = 2 * b.R / kFillSlots + (i64)b.N * strips * (64 * kStripCols / kFillSlots + 1) + 1;
     if (waves > 8192) waves = 8192;
     CWR_LAUNCH(k_fill, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, b.stream, b.lx, b.ly, b.row_off,
                        ws.pad_off, ws.fill_off, ws.seqmode, b.N, b.R, ws.lp.l, ws.alpha, ws.beta, ws.scale_a,

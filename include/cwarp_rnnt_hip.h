@@ -97,7 +97,8 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
  *      walk carries); bit 1 / bit 2 = alpha / beta was walked again in the log domain.  A sequence
  *      with more than 8 strips of 128 labels is always in the log domain.
  *   5  scale_a, 6  scale_b: int32 scale exponents of the linear-domain walk
- * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U).
+ * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U): row
+ * t + (u%128)/2 + 64 of its strip, whose rows are nl rounded up to even slots apart.
  * Log-domain values are base-2 logarithms (multiply by ln 2).  Linear-domain values are
  * value * 2^C: a strip s = u/128 of width nl = min(128, U+1-128s) is walked by L = ceil(nl/2) lanes,
  * lane l = (u%128)/2 holding columns 2l and 2l+1; the walk step is k = t+l (alpha) or

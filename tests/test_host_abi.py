@@ -68,7 +68,8 @@ def test_workspace_size_is_monotone_and_bounded():
 def test_lattice_slot_is_a_bijection_into_the_bound():
     """Every cell of a T x (U+1) lattice gets its own slot below the lattice size, for shapes around
     the 128-column strip width (two columns per lane: even and odd widths), and the two cells of a
-    lane lie next to each other in one strip row."""
+    lane lie next to each other in one strip row, on a 16-byte boundary of an array of 8-byte
+    records (rows are an even number of slots apart: a strip of odd width has a column of padding)."""
     lib = _lib.load()
     for T, U in [(1, 0), (1, 70), (5, 3), (3, 126), (3, 127), (3, 128), (2, 260), (40, 129), (7, 4)]:
         slots = set()
@@ -79,11 +80,13 @@ def test_lattice_slot_is_a_bijection_into_the_bound():
                 slots.add(s)
                 if u % 2 == 1:
                     assert s == lib.cwr_lattice_slot(t, u - 1, T, U) + 1
+                else:
+                    assert s % 2 == 0
         assert len(slots) == T * (U + 1)
         strips = U // 128 + 1
         nl = U + 1 - 128 * (strips - 1)
         lanes = (nl + 1) // 2
-        size = (strips - 1) * (T + 63 + 64) * 128 + (T + lanes - 1 + 64) * nl
+        size = (strips - 1) * (T + 63 + 64) * 128 + (T + lanes - 1 + 64) * 2 * lanes
         assert max(slots) < size
         assert lib.cwr_lattice_slot(T, 0, T, U) == -1 and lib.cwr_lattice_slot(0, U + 1, T, U) == -1
 
