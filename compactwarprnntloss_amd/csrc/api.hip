@@ -372,7 +372,8 @@ int cwr_joint_forward_fg(const void* f, const void* g, int act, int64_t T_pad, i
     if (dtype != CWR_F16 && dtype != CWR_BF16) return CWR_ERR_DTYPE;
     if (act < CWR_ACT_NONE || act > CWR_ACT_RELU) return CWR_ERR_MODE;
     // the joint sizes whose rows a wave keeps in registers
-    if (H != 256 && H != 384 && H != 512 && H != 640 && H != 768 && H != 1024) return CWR_ERR_SHAPE;
+    // the joint sizes whose rows a wave keeps in registers
+    if (H % 64 != 0 || H < 128 || H > 1024) return CWR_ERR_SHAPE;
     if (T_pad < 0 || Up_pad < 0) return CWR_ERR_SHAPE;
     if (T_pad > 0x3fffffff || Up_pad > 0x3fffffff) return CWR_ERR_TOO_LARGE;
     if (R > 0 && (!f || !g || !w)) return CWR_ERR_NULL;

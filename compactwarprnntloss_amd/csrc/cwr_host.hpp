@@ -40,7 +40,7 @@ struct Workspace {
     i64* fill_off;  // N+1  first chunk of each sequence in k_fill's work list (a running sum: searchable)
     i64* bnd_off;   // N+1  first boundary-stream entry of each sequence
     int* seqmode;   // N+1  per sequence: 0 = walked in the scaled linear domain; bit 0 = in the log domain
-                    //      (gather's verdict), bits 1 / 2 = alpha / beta repeated in the log domain
+                    //      (set by the gather pass), bits 1 / 2 = alpha / beta repeated in the log domain
     LpStore lp;     // 2 x slot_cap  gathered (blank, label) probabilities and log-probabilities
     double* alpha;  // slot_cap  log2(alpha), or alpha * 2^scale_a[block][column] (see seqmode)
     double* beta;   // slot_cap

@@ -651,7 +651,7 @@ __device__ __forceinline__ void join_resident_rows_as(const JoinSrc<T>& s, i64 R
         // in; g's follow in batches of kBatch into spare registers and each batch is folded in as it
         // arrives.  (One fragment of each at a time, which is what the loop would otherwise compile
         // to, pays a trip to the L2 per fragment: 32 of them in a row at H = 512.)
-        constexpr int kBatch = KS >= 24 ? 4 : 8;  // the longer the resident row, the fewer spare registers
+        constexpr int kBatch = (KS >= 24 || KS % 8 != 0) ? 4 : 8;  // the longer the resident row, the fewer spare registers
         static_assert(KS % kBatch == 0, "whole batches");
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) hreg[nd][ks] = *reinterpret_cast<const v4i*>(pf + 16 * ks);
@@ -880,10 +880,18 @@ __global__ __launch_bounds__(64 * WAVES, OCC) void k_joint_dz_res(
 //   spill), tiles of 64 entries 0.49 ms (half the LDS reads per matrix instruction, but a lone wave
 //   per SIMD hides neither the LDS latency nor the tile's reduction); streaming kernel 0.63 ms.
 //   the backward kernel follows, except at H = 512 (0.61 against 0.57 ms: it keeps four waves).
-#define CWR_JOINT_SHAPES(X) X(1, 16, 4, 8, 64, 1, true) X(1, 24, 4, 8, 64, 1, true) X(1, 32, 4, 8, 64, 1, false) \
-                            X(1, 40, 4, 8, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 64, 4, 4, 64, 1, true)
-#define CWR_JOINT_DZ_SHAPES(X) X(1, 16, 4, 8, 64, 1, true) X(1, 24, 4, 8, 64, 1, true) X(1, 32, 4, 4, 64, 2, false) \
-                               X(1, 40, 4, 8, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 64, 4, 4, 64, 1, true)
+//   the other multiples of 64 from 128 to 1024 take the shape of their larger neighbour,
+//   with one register set of weight loads where the number of K-slices per tile is odd.
+#define CWR_JOINT_SHAPES(X) X(1, 8, 4, 8, 64, 1, true) X(1, 12, 4, 8, 64, 1, false) X(1, 16, 4, 8, 64, 1, true) \
+                            X(1, 20, 4, 8, 64, 1, false) X(1, 24, 4, 8, 64, 1, true) X(1, 28, 4, 8, 64, 1, false) \
+                            X(1, 32, 4, 8, 64, 1, false) X(1, 36, 4, 8, 64, 1, false) X(1, 40, 4, 8, 64, 1, false) \
+                            X(1, 44, 4, 4, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 52, 4, 4, 64, 1, false) \
+                            X(1, 56, 4, 4, 64, 1, true) X(1, 60, 4, 4, 64, 1, false) X(1, 64, 4, 4, 64, 1, true)
+#define CWR_JOINT_DZ_SHAPES(X) X(1, 8, 4, 8, 64, 1, true) X(1, 12, 4, 8, 64, 1, false) X(1, 16, 4, 8, 64, 1, true) \
+                               X(1, 20, 4, 8, 64, 1, false) X(1, 24, 4, 8, 64, 1, true) X(1, 28, 4, 4, 64, 2, false) \
+                               X(1, 32, 4, 4, 64, 2, false) X(1, 36, 4, 8, 64, 1, false) X(1, 40, 4, 8, 64, 1, false) \
+                               X(1, 44, 4, 4, 64, 1, false) X(1, 48, 4, 4, 64, 1, true) X(1, 52, 4, 4, 64, 1, false) \
+                            X(1, 56, 4, 4, 64, 1, true) X(1, 60, 4, 4, 64, 1, false) X(1, 64, 4, 4, 64, 1, true)
 
 template <typename T>
 static int joint_gather_typed(const Batch& b, const Workspace& ws, const JointOperands& j, float* lse, int* rowinfo,

@@ -10,11 +10,11 @@
 // walks it along skewed diagonals; at step q lane l holds the cells (t = q - l, u = 128 s + 2l) and
 // (t, u + 1).  The neighbour in u of the lane's first column is the adjacent lane (one DPP wave
 // shift), that of its second column the lane itself, the neighbour in t is the lane's own previous
-// value, so a step needs no barrier.  A lone wave issues one instruction every four to five cycles
-// whatever its kind, so the step is written for the smallest instruction count:
+// value, so a step needs no barrier.  A lone wave pays five to nine clocks for every instruction
+// it issues, whatever its kind, so the step is written for the smallest instruction count:
 //   - the strip layout (see lattice_slot) makes every step's access one row at a constant pitch:
-//     buffer instructions with a per-lane constant offset and a scalar row offset, no address
-//     arithmetic on the vector unit;
+//     buffer instructions with a per-lane constant offset and a scalar row offset that never
+//     changes (the block's position sits in the descriptor), no address arithmetic at all;
 //   - no lane is ever predicated: lanes that hold no cell read and write padding slots, and the
 //     recursion keeps them at the "no path" marker by itself (see below);
 //   - the normal number system is the scaled linear domain (one fp64 add and two multiplies per
@@ -415,9 +415,10 @@ __device__ __forceinline__ double place_entry(double nbr, double e, int j) {
 // C renewed at the start of every block of kPF steps so that the largest of the lane's own values
 // and of what its neighbour is about to hand over sits at 2^kLinTarget.  A value arriving from the
 // neighbouring lane is brought to the lane's scale by the (block-constant) power of two that
-// separates the two scales, inside the multiply-add that takes it in.  Like a logarithm, this loses nothing across lanes, however far
-// apart their magnitudes are: the only thing that can underflow is a summand that is negligible
-// next to the other summand of the SAME cell, or one of a lane's two columns next to the other.
+// separates the two scales, inside the multiply-add that takes it in.  Like a logarithm, this
+// loses nothing across lanes, however far apart their magnitudes are: the only thing that can
+// underflow is a summand that is negligible next to the other summand of the SAME cell, or one of
+// a lane's two columns next to the other.
 // Within a block a lane's value can still drift out of the fp64 range (a run of extreme factors,
 // or a much larger magnitude arriving from several columns away), which the range check catches.
 // In a strip of odd width the last lane's second column is the layout's column of padding: zero
@@ -885,7 +886,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(
     none.slots = nullptr; none.scales = nullptr; none.produced = nullptr; none.consumed = nullptr;
 
     const bool concurrent = S <= W;
-    const bool linear = concurrent && (seqmode[n] & 1) == 0;  // the gather pass's verdict on the log-probs
+    const bool linear = concurrent && (seqmode[n] & 1) == 0;  // what the gather pass found about the log-probs
     if (concurrent) {
         // position p in the order of the walk: alpha strip p, beta strip S-1-p
         const bool active = w < S;

@@ -116,7 +116,7 @@ def rnnt_forward(xs, lx, ys, ly, blank: int, fused: bool, max_u: Optional[int] =
     return costs, st
 
 
-RESIDENT_JOINT_SIZES = (256, 384, 512, 640, 768, 1024)  # joint sizes whose rows a wave keeps in registers
+RESIDENT_JOINT_SIZES = tuple(range(128, 1025, 64))  # joint sizes whose rows a wave keeps in registers
 
 
 def _joint_state(like, weight, bias, lx, ys, ly, R: int, max_u: Optional[int]):

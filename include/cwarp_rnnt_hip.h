@@ -286,7 +286,9 @@ int cwr_join_backward(const void* dh, const void* h, int dtype, int act, int64_t
  * CWR_MODE_FUSED would run on stored logits, and removes the (R, V) logits from memory.
  *   h     (R, H) compact joint activations (e.g. from cwr_join), w (V, H) output-layer weight (the
  *         layout of a torch.nn.Linear weight), both of `dtype` = CWR_F16 or CWR_BF16, contiguous,
- *         16-byte aligned;  H a multiple of 32
+ *         16-byte aligned;  H a multiple of 32 (a multiple of 64 from 128 to 1024 is read exactly
+ *         once, every wave keeping its rows in registers; any other size is streamed once per tile
+ *         of 128 vocabulary entries, at less than half the speed)
  *   bias  (V,) fp32 or NULL
  * All other arguments and every output as for cwr_forward with mode = CWR_MODE_FUSED; lse, rowinfo
  * and grads are what cwr_joint_backward reads. */
@@ -303,7 +305,7 @@ int cwr_joint_forward(const void* h, const void* w, const float* bias, int dtype
  * exist in memory.  The reference repository has no joiner (see cwr_join).
  *   f (N, T_pad, H), g (N, Up_pad, H), w (V, H) of `dtype` = CWR_F16 or CWR_BF16, contiguous, 16-byte
  *         aligned;  act a cwr_activation
- *   H     one of 256, 384, 512, 640, 768, 1024 (the sizes whose rows a wave keeps in registers);
+ *   H     a multiple of 64 from 128 to 1024 (the sizes whose rows a wave keeps in registers);
  *         any other H: CWR_ERR_SHAPE, and the caller runs cwr_join + cwr_joint_forward instead
  *   h_out (R, H) or NULL: receives the joint rows, bit-identical to cwr_join's, for a backward pass
  *         that needs them (cwr_joint_backward, the weight-gradient product, cwr_join_backward)

@@ -43,6 +43,15 @@ def reference(j, grad_out=None, want_dense=False):
     ([30, 14], [9, 3], 32, 40, True),                     # fewer entries than half a tile: a wave with no valid entry
     ([61, 40], [33, 70], 512, 1000, True),                # the largest resident shape at two waves per SIMD
     ([25, 31], [20, 9], 768, 257, False),                 # one wave per SIMD, a single odd entry in the last tile
+    ([33, 12], [8, 40], 128, 300, True),                  # two K-slices per vocabulary tile
+    ([33, 12], [8, 40], 192, 257, False),                 # an odd number of K-slices per tile (3)
+    ([20, 41], [30, 6], 320, 1024, True),                 # ... 5
+    ([27, 9], [11, 25], 448, 130, True),                  # ... 7
+    ([27, 9], [11, 25], 576, 515, False),                 # ... 9
+    ([18, 22], [14, 9], 896, 300, True),                  # one wave per SIMD, 14 slices
+    ([18, 22], [14, 9], 704, 130, False),                 # one wave per SIMD, odd numbers of slices
+    ([11, 15], [9, 14], 832, 257, True),
+    ([11, 15], [9, 14], 960, 64, True),
 ])
 def test_joint_forward_matches_oracle(dtype, lx, ly, H, V, bias):
     import compactwarprnntloss_amd as pkg
@@ -73,6 +82,9 @@ def test_joint_forward_matches_oracle(dtype, lx, ly, H, V, bias):
     ([50, 21], [30, 70], 256, 1024, False, 77),           # resident kernel, two data blocks per wave
     ([50, 21], [30, 20], 512, 515, True, 130),            # resident kernel; V not a multiple of 4: element stores
     ([30, 14], [9, 3], 32, 40, True, 5),
+    ([33, 12], [8, 40], 192, 257, True, 3),               # an odd number of K-slices per tile
+    ([27, 9], [11, 25], 448, 130, False, 129),            # ... in the four-wave shape
+    ([18, 22], [14, 9], 896, 300, True, 0),
 ])
 def test_joint_backward_dlogits_match_oracle(dtype, lx, ly, H, V, bias, blank):
     """cwr_joint_backward through the C ABI, a block of rows at a time (blocks that end inside a
@@ -212,7 +224,7 @@ def test_joint_random_shapes_against_oracle(seed):
         N = int(rng.integers(65, 80)) if rng.random() < 0.15 else int(rng.integers(1, 6))
         lx = rng.integers(1, 40 if N < 10 else 6, N)
         ly = rng.integers(0, 80 if (N < 10 and rng.random() < 0.3) else 12, N)
-        H = int(rng.choice([32, 64, 96, 256, 384, 512, 640, 768, 1024]))
+        H = int(rng.choice([32, 64, 96] + list(range(128, 1025, 64))))
         V = int(rng.choice([5, 40, 128, 130, 256, 300, 515, 1024]))
         dtype = str(rng.choice(["bf16", "f16"]))
         blank = int(rng.integers(0, V))
@@ -383,7 +395,10 @@ def make_fg(lx, ly, H, seed, dtype, T_extra=2, U_extra=1):
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("act", [None, "tanh", "relu"])
 @pytest.mark.parametrize("lx,ly,H,V", [([9, 5, 12, 1], [3, 0, 7, 4], 256, 128), ([40, 33, 17], [12, 20, 5], 512, 300),
-                                       ([25, 31], [20, 9], 768, 257), ([14, 6], [5, 130], 384, 64)])
+                                       ([25, 31], [20, 9], 768, 257), ([14, 6], [5, 130], 384, 64),
+                                       ([12, 9], [7, 20], 128, 130), ([12, 9], [7, 20], 192, 64),
+                                       ([21, 8], [6, 33], 320, 300), ([21, 8], [6, 33], 448, 64),
+                                       ([16, 10], [12, 5], 576, 257), ([16, 10], [12, 5], 896, 130)])
 def test_joiner_chain_forward_matches_oracle(dtype, act, lx, ly, H, V):
     """cwr_joint_forward_fg: rows act(f[n,t] + g[n,u]) formed in the kernel.  Oracle: join_rows in
     float64, rounded once to the 16-bit type (the kernel's one rounding), joint_logits, fused-mode
