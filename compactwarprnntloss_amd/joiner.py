@@ -120,6 +120,20 @@ class _JointLoss(torch.autograd.Function):
         return dh, dw, db, None, None, None, None, None, None, None, None
 
 
+_BLOCK_BYTES = 384 << 20   # logit gradients alive at a time when the caller sets no block size
+_BLOCK_MIN_ROWS = 65536    # fewer rows than this no longer fill the GPU with 128-row workgroups
+
+
+def _balanced_block(R: int, V: int, itemsize: int) -> int:
+    """Rows per block of the backward pass: the fewest blocks of at most _BLOCK_BYTES of logit
+    gradients, all of the same size (a short last block runs the matrix kernels at a fraction of
+    their speed: N=32, V=1024, H=512, R=311449: 131072 + 131072 + 49305 rows 1.97 ms forward +
+    backward, two blocks of 155725 rows 1.83 ms, one block 1.74 ms)."""
+    limit = max(_BLOCK_MIN_ROWS, _BLOCK_BYTES // max(1, V * itemsize))
+    blocks = max(1, -(-R // limit))
+    return max(1, (-(-R // blocks) + 255) // 256 * 256)
+
+
 def _joint_backward(h, weight, bias, st, grad_out, reduction, blank, chunk_rows):
     """(dh, dW, dbias) of the loss of logits = h @ weight.T + bias from the state its forward call left:
     cwr_joint_backward a block of rows at a time, library GEMMs on each block."""
@@ -136,7 +150,7 @@ def _joint_backward(h, weight, bias, st, grad_out, reduction, blank, chunk_rows)
     dw = torch.zeros((V, H), dtype=torch.float32, device=dev)
     db = torch.zeros(V, dtype=torch.float32, device=dev) if bias is not None else None
     bias_f = bias.to(torch.float32).contiguous() if bias is not None else None
-    chunk = max(1, min(int(chunk_rows), R))
+    chunk = max(1, min(int(chunk_rows), R)) if chunk_rows > 0 else _balanced_block(R, V, h.element_size())
     z = torch.empty((chunk, V), dtype=h.dtype, device=dev)
     with torch.cuda.device(dev):
         stream = _stream_ptr(dev)
@@ -215,7 +229,7 @@ def fused_joiner_loss(f: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, bi
                       lx: torch.Tensor, y: torch.Tensor, ly: torch.Tensor, blank: int = 0,
                       reduction: Optional[str] = "mean", activation: Optional[str] = "tanh", *,
                       total_rows: Optional[int] = None, max_u: Optional[int] = None, validate: bool = False,
-                      chunk_rows: int = 131072, one_kernel: Optional[bool] = None) -> torch.Tensor:
+                      chunk_rows: Optional[int] = None, one_kernel: Optional[bool] = None) -> torch.Tensor:
     """transducer_loss of the logits act(f[n,t] + g[n,u]) @ weight.T + bias, the joiner's whole chain,
     with neither the (R, H) joint rows nor the (R, V) logits in memory on the way to the loss: f
     (N, T, H) encoder frames and g (N, U+1, H) predictor states projected to the joint space, weight
@@ -245,22 +259,23 @@ def fused_joiner_loss(f: torch.Tensor, g: torch.Tensor, weight: torch.Tensor, bi
                                 chunk_rows=chunk_rows)
     return _JoinerLoss.apply(f.contiguous(), g.contiguous(), weight.contiguous(), bias, lx, y, ly, int(blank),
                              reduction if reduction in ("mean", "sum") else "none", _ACTS[activation],
-                             int(total_rows), max_u, bool(validate), int(chunk_rows))
+                             int(total_rows), max_u, bool(validate), -1 if chunk_rows is None else int(chunk_rows))
 
 
 def fused_joint_loss(h: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], lx: torch.Tensor,
                      y: torch.Tensor, ly: torch.Tensor, blank: int = 0, reduction: Optional[str] = "mean", *,
-                     max_u: Optional[int] = None, validate: bool = False, chunk_rows: int = 131072) -> torch.Tensor:
+                     max_u: Optional[int] = None, validate: bool = False, chunk_rows: Optional[int] = None) -> torch.Tensor:
     """transducer_loss(h @ weight.T + bias, lx, y, ly, blank, reduction, fused_log_softmax=True) without
     the (R, V) logits: h (R, H) compact joint activations (e.g. from compact_join), weight (V, H) and
     bias (V,) or None the output layer, fp16 or bf16.  Differentiable in h, weight and bias; the
-    backward pass holds at most chunk_rows x V logits at a time."""
+    backward pass holds at most chunk_rows x V logit gradients at a time (None: equal blocks of at
+    most 384 MiB each)."""
     assert lx.dtype == torch.int32 and ly.dtype == torch.int32 and y.dtype == torch.int32
     assert reduction in ["mean", "sum", "none"] or reduction is None
     assert blank >= 0 and blank < weight.size(0)
     return _JointLoss.apply(h.contiguous(), weight.contiguous(), bias, lx, y, ly, int(blank),
                             reduction if reduction in ("mean", "sum") else "none", max_u, bool(validate),
-                            int(chunk_rows))
+                            -1 if chunk_rows is None else int(chunk_rows))
 
 
 class CompactJoiner(torch.nn.Module):
