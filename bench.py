@@ -109,7 +109,7 @@ def main():
                          "batch's storage type) and its backward at the same lengths (reported under 'joiner_op'; "
                          "not part of 'value')")
     ap.add_argument("--with-long-labels", action="store_true",
-                    help="also time the forward call and its lattice stage on N=4, T=1250 and U = 300 ... 1200 labels "
+                    help="also time the forward call and its lattice stage on N=4, T=1250 and U = 300 ... 2300 labels "
                          "(log-prob mode, V=4: the lattice dominates; reported under 'long_labels')")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so that a counter run can scale "
@@ -267,7 +267,7 @@ def main():
         import ctypes as C
         lib = pkg._lib.load()
         rows = []
-        for U in (300, 511, 600, 1000, 1023, 1200):
+        for U in (300, 511, 600, 1000, 1023, 1200, 2000, 2300):
             Nl, Tl, Vl = 4, 1250, 4
             lxl = torch.full((Nl,), Tl, dtype=torch.int32, device=dev)
             lyl = torch.full((Nl,), U, dtype=torch.int32, device=dev)

@@ -841,31 +841,33 @@ __device__ __forceinline__ void log_dispatch(bool has_in, bool has_out, int T, i
 // demands plus one block of kPF steps of slack; the boundary values travel through LDS rings
 // guarded by two progress counters per ring.  A wave only ever waits for the wave of the strip
 // before it (values) or after it (ring space), and the first strip waits for nobody, so the chain
-// always drains; every wait is bounded all the same.  Longer sequences (S > W, 1024 labels or more)
+// always drains; every wait is bounded all the same.  Longer sequences (S > W, 2048 labels or more)
 // fall back to one wave walking the strips in turn, in the log domain, with the streams in global
 // memory.
-constexpr int kMaxWaves = 8;
+constexpr int kMaxWaves = 16;  // strips of a sequence that are ever walked at once
 
-// At most two waves of this kernel share a SIMD (eight waves per workgroup, one workgroup per CU is
-// all a batch ever needs), which lets a wave keep both prefetch rings and the walk's state in up to
-// 256 registers; at the default budget of 128 the register allocator rotates the rings through
-// copies that wait for loads in flight and a step takes twice as long.
-__global__ __launch_bounds__(kMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(1, 2))) void k_lattice(
+// Two shapes.  Up to eight strips (label sequences below 1024, all a batch normally holds): at most
+// two waves share a SIMD, which lets a wave keep the prefetch ring and the walk's state in up to
+// 256 registers.  Nine to sixteen strips: sixteen waves per workgroup, four per SIMD, 128 registers
+// each; the host picks the shape from the max_u of the call, so a sequence of S <= 16 strips
+// always finds S waves.
+template <int MAXW>
+__global__ __launch_bounds__(MAXW * 64) __attribute__((amdgpu_waves_per_eu(1, MAXW / 4))) void k_lattice(
     const int* __restrict__ lx, const int* __restrict__ ly, const i64* __restrict__ pad_off,
     const i64* __restrict__ bnd_off, int* seqmode, const LpStore lp, double* alpha,
     double* beta, int* scale_a, int* scale_b, double* bnd_a, double* bnd_b, int beta_only, int spin_limit,
     int* status_word) {
-    __shared__ double s_ring[kMaxWaves - 1][2 * kRing + 64];
-    __shared__ int s_scale[kMaxWaves - 1][kRing / kPF];
-    __shared__ int s_produced[kMaxWaves];
-    __shared__ int s_consumed[kMaxWaves];
+    __shared__ double s_ring[MAXW - 1][2 * kRing + 64];
+    __shared__ int s_scale[MAXW - 1][kRing / kPF];
+    __shared__ int s_produced[MAXW];
+    __shared__ int s_consumed[MAXW];
     __shared__ volatile int s_unsafe;
     __shared__ int s_abort;
     const int n = blockIdx.x;
     const int dir = beta_only ? 1 : (int)blockIdx.y;
     const int W = blockDim.x >> 6;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    if (threadIdx.x < kMaxWaves) {
+    if (threadIdx.x < MAXW) {
         s_produced[threadIdx.x] = 0;
         s_consumed[threadIdx.x] = 0;
     }
@@ -967,9 +969,15 @@ static int lattice_waves(const Batch& b) {
 int launch_lattice(const Batch& b, const Workspace& ws, bool beta_only) {
     if (b.N == 0) return CWR_OK;
     dim3 grid((unsigned)b.N, beta_only ? 1 : 2);
-    CWR_LAUNCH(k_lattice, grid, dim3(lattice_waves(b) * 64), 0, b.stream, b.lx, b.ly, ws.pad_off,
-                       ws.bnd_off, ws.seqmode, ws.lp, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, ws.bnd_a,
-                       ws.bnd_b, beta_only ? 1 : 0, wait_limit(), b.status);
+    const int waves = lattice_waves(b);
+    if (waves <= 8)
+        CWR_LAUNCH(k_lattice<8>, grid, dim3(waves * 64), 0, b.stream, b.lx, b.ly, ws.pad_off, ws.bnd_off, ws.seqmode,
+                   ws.lp, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, ws.bnd_a, ws.bnd_b, beta_only ? 1 : 0,
+                   wait_limit(), b.status);
+    else
+        CWR_LAUNCH(k_lattice<16>, grid, dim3(waves * 64), 0, b.stream, b.lx, b.ly, ws.pad_off, ws.bnd_off, ws.seqmode,
+                   ws.lp, ws.alpha, ws.beta, ws.scale_a, ws.scale_b, ws.bnd_a, ws.bnd_b, beta_only ? 1 : 0,
+                   wait_limit(), b.status);
     return check_launch();
 }
 

@@ -95,7 +95,7 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
  *   4  seqmode: N+1 int32 (N used), how the sequence was walked.  0 = both directions in the
  *      scaled linear domain; bit 0 = both in the log domain (log-probs outside what the linear
  *      walk carries); bit 1 / bit 2 = alpha / beta was walked again in the log domain.  A sequence
- *      with more than 8 strips of 128 labels is always in the log domain.
+ *      with more than 16 strips of 128 labels is always in the log domain.
  *   5  scale_a, 6  scale_b: int32 scale exponents of the linear-domain walk
  * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U): row
  * t + (u%128)/2 + 64 of its strip, whose rows are nl rounded up to even slots apart.

@@ -40,7 +40,8 @@ def _lp_of(b, n, fused):
     ([9, 5, 12, 1], [3, 0, 7, 4], 1.0),          # small, ragged, U=0 and T=1
     ([40, 150], [70, 130], 1.0),                 # one and two strips of 128 labels
     ([30, 7, 20], [20, 600, 300], 1.0),          # five and three strips, walked concurrently
-    ([6, 9], [1100, 40], 1.0),                   # nine strips: the sequential log-domain walk
+    ([6, 9], [1100, 40], 1.0),                   # nine strips, walked concurrently by sixteen waves
+    ([3, 5], [2100, 10], 1.0),                   # seventeen strips: the sequential log-domain walk
     ([60, 33], [25, 64], 40.0),                  # steep logits: the per-sequence log-domain walk
 ])
 def test_alpha_beta_export_matches_oracle(fused, lx, ly, sigma):
