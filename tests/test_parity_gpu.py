@@ -762,3 +762,49 @@ def test_random_hard_regimes_against_oracle(seed):
         except AssertionError as err:
             raise AssertionError(f"seed {seed} case {case} ({kind}): N={N} lx={lx.tolist()} ly={ly.tolist()} V={V} "
                                  f"{dtype} fused={fused} blank={blank} sigma={sigma}\n{err}")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_small_batches_against_the_c_restatement(seed):
+    """Four hundred small random batches per seed (one to six sequences, 1 to 120 frames, 0 to 300
+    labels so that strips of every width and up to three strips occur, V from 3 to 32, both modes,
+    logits of scale 0.5 to 12, some rows peaked, any blank) through the forward call, against the C
+    restatement of the oracle (pinned to the NumPy oracle in tests/test_oracle_pins.py): costs within
+    1e-5 relative + 1e-6 absolute, per-row gradients within 1e-4, no flag raised."""
+    from oracle import build_c
+    lib = build_c.load()
+    pkg = _pkg()
+    dev = torch.device("cuda:0")
+    for case in range(400):
+        rng = np.random.default_rng(7700000 + 1000 * seed + case)
+        N = int(rng.integers(1, 7))
+        kind = int(rng.integers(0, 4))
+        tmax, umax = [(6, 4), (40, 70), (120, 140), (30, 300)][kind]
+        lx = rng.integers(1, tmax + 1, N).astype(np.int32)
+        ly = rng.integers(0, umax + 1, N).astype(np.int32)
+        if rng.random() < 0.2:
+            ly[rng.integers(0, N)] = 0
+        if rng.random() < 0.2:
+            lx[rng.integers(0, N)] = 1
+        V = int(rng.choice([3, 4, 8, 17, 32]))
+        fused = bool(rng.integers(0, 2))
+        sigma = float(rng.choice([0.5, 1.0, 2.0, 5.0, 12.0]))
+        R = int((lx.astype(np.int64) * (ly + 1)).sum())
+        x = (rng.standard_normal((R, V)) * sigma).astype(np.float32)
+        if rng.random() < 0.15:
+            x[np.arange(R), rng.integers(0, V, R)] += 30.0
+        if not fused:
+            x = orc.log_softmax(x.astype(np.float64)).astype(np.float32)
+        blank = int(rng.integers(0, V))
+        yp = np.zeros((N, max(int(ly.max()), 1)), dtype=np.int32)
+        for n in range(N):
+            lab = rng.integers(0, V - 1, int(ly[n])).astype(np.int32)
+            lab[lab >= blank] += 1
+            yp[n, : ly[n]] = lab
+        ref = build_c.loss_and_grad(lib, x, lx, yp, ly, blank, fused, None, want_G=True, want_grad=False)
+        costs, st = pkg.rnnt_forward(torch.from_numpy(x).to(dev), torch.from_numpy(lx).to(dev),
+                                     torch.from_numpy(yp).to(dev), torch.from_numpy(ly).to(dev), blank, fused)
+        what = f"seed {seed} case {case}: lx={lx.tolist()} ly={ly.tolist()} V={V} fused={fused} sigma={sigma} blank={blank}"
+        assert int(st.status[0].item()) == 0, what
+        np.testing.assert_allclose(costs.cpu().numpy(), ref["costs"], rtol=LOSS_RTOL, atol=1e-6, err_msg=what)
+        np.testing.assert_allclose(st.grads.cpu().numpy(), ref["G"], rtol=0, atol=GRAD_ATOL, err_msg=what)
