@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("CWARP_RNNT_LIB") or os.path.join(HERE, "libcwarp_rnnt
 # enum cwr_dtype / cwr_mode / cwr_flag
 F32, F16, BF16, F64 = 0, 1, 2, 3
 MODE_LOGPROB, MODE_FUSED = 0, 1
-NOALLOC_SCRATCH_BYTES = 96 << 20  # CWR_NOALLOC_SCRATCH_BYTES
+NOALLOC_SCRATCH_BYTES = 128 << 20  # CWR_NOALLOC_SCRATCH_BYTES
 FLAG_ROWS_MISMATCH, FLAG_BAD_LENGTH, FLAG_BAD_LABEL, FLAG_FB_MISMATCH, FLAG_U_TOO_LARGE, FLAG_INTERNAL = \
     1, 2, 4, 8, 16, 32
 FLAG_NAMES = {

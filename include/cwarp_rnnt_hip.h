@@ -98,7 +98,7 @@ size_t cwr_workspace_bytes(int64_t N, int64_t R, int64_t max_u);
  *      with more than 16 strips of 128 labels is always in the log domain.
  *   5  scale_a, 6  scale_b: int32 scale exponents of the linear-domain walk
  * Cell (t,u) of sequence n lives at element pad_off[n] + cwr_lattice_slot(t,u,T,U): row
- * t + (u%128)/2 + 64 of its strip, whose rows are nl rounded up to even slots apart.
+ * t + (u%128)/2 + 32 of its strip, whose rows are nl rounded up to even slots apart.
  * Log-domain values are base-2 logarithms (multiply by ln 2).  Linear-domain values are
  * value * 2^C: a strip s = u/128 of width nl = min(128, U+1-128s) is walked by L = ceil(nl/2) lanes,
  * lane l = (u%128)/2 holding columns 2l and 2l+1; the walk step is k = t+l (alpha) or
@@ -154,10 +154,10 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
  * CWR_NOALLOC_SCRATCH_BYTES inside the library's device code, one copy per GPU, there for as long as
  * the process lives.  The call makes no allocation of any kind.
  *   - cwr_workspace_bytes(N, R, max_u) must not exceed CWR_NOALLOC_SCRATCH_BYTES, else
- *     CWR_ERR_TOO_LARGE.  96 MiB: the N=32, T~175, U~50 batch (R = 3.1e5) needs 30 MiB, the
- *     long-form N=4, T~1250, U~300 batch (R = 1.5e6) 71 MiB.
+ *     CWR_ERR_TOO_LARGE.  128 MiB: the N=32, T~175, U~50 batch (R = 3.1e5) needs 39 MiB, the
+ *     long-form N=4, T~1250, U~300 batch (R = 1.5e6) 119 MiB.
  *   - The array is part of the library's device code: every process that loads the library holds
- *     96 MiB on every GPU it runs the library's kernels on, whether or not it ever calls this entry
+ *     128 MiB on every GPU it runs the library's kernels on, whether or not it ever calls this entry
  *     point.
  *   - The first call on a GPU looks the array's address up (hipGetSymbolAddress); make it outside
  *     a stream capture.  Calls with arguments the host can reject (null or misaligned pointers, bad
@@ -167,7 +167,7 @@ int cwr_forward(const void* x, int dtype, int64_t R, int64_t V,
  *     call is relied on, the kernels initialise what they read.
  *   - The array holds the lattice state of the LAST call on that GPU only; cwr_export_lattice does
  *     not reach it. */
-#define CWR_NOALLOC_SCRATCH_BYTES (96u << 20)
+#define CWR_NOALLOC_SCRATCH_BYTES (128u << 20)
 int cwr_forward_noalloc(const void* x, int dtype, int64_t R, int64_t V,
                         const int32_t* lx, const int32_t* ly, const int32_t* y, int64_t y_stride, int64_t y_len,
                         int64_t N, int32_t blank, int mode, int64_t max_u,
