@@ -380,41 +380,43 @@ def main():
                 z = torch.nn.functional.linear(hj, Wj, bj)
             pkg.rnnt_forward(z, lx, y, ly, 0, True, max_u=y.size(1))
 
-        # The joiner's whole chain (broadcast sum + tanh + output layer + loss) as one kernel against
-        # its two-kernel form (cwr_join, then cwr_joint_forward on the stored rows), same lengths.
-        Tm, Up = int(cfg["lx"].max()), int(cfg["ly"].max()) + 1
-        fj = torch.randn((N, Tm, H), device=dev).to(jd)
-        gj = torch.randn((N, Up, H), device=dev).to(jd)
-        chain_fwd = timed(lambda: pkg.loss.joint_forward_fg(fj, gj, 1, Wj, bj, lx, y, ly, 0, R, max_u=y.size(1)))
-        chain_fwd_keep = timed(lambda: pkg.loss.joint_forward_fg(fj, gj, 1, Wj, bj, lx, y, ly, 0, R, max_u=y.size(1),
-                                                                 keep_rows=True))
+        joiner_chain = None  # the one-kernel form exists for the joint sizes whose rows stay in registers
+        if H in pkg.loss.RESIDENT_JOINT_SIZES:
+            # The joiner's whole chain (broadcast sum + tanh + output layer + loss) as one kernel against
+            # its two-kernel form (cwr_join, then cwr_joint_forward on the stored rows), same lengths.
+            Tm, Up = int(cfg["lx"].max()), int(cfg["ly"].max()) + 1
+            fj = torch.randn((N, Tm, H), device=dev).to(jd)
+            gj = torch.randn((N, Up, H), device=dev).to(jd)
+            chain_fwd = timed(lambda: pkg.loss.joint_forward_fg(fj, gj, 1, Wj, bj, lx, y, ly, 0, R, max_u=y.size(1)))
+            chain_fwd_keep = timed(lambda: pkg.loss.joint_forward_fg(fj, gj, 1, Wj, bj, lx, y, ly, 0, R, max_u=y.size(1),
+                                                                     keep_rows=True))
 
-        def two_kernel_fwd():
-            hh = pkg.compact_join(fj, gj, lx, ly, "tanh", total_rows=R)
-            pkg.joint_forward(hh, Wj, bj, lx, y, ly, 0, max_u=y.size(1))
+            def two_kernel_fwd():
+                hh = pkg.compact_join(fj, gj, lx, ly, "tanh", total_rows=R)
+                pkg.joint_forward(hh, Wj, bj, lx, y, ly, 0, max_u=y.size(1))
 
-        two_fwd = timed(two_kernel_fwd)
-        fp, gp = fj.clone().requires_grad_(True), gj.clone().requires_grad_(True)
+            two_fwd = timed(two_kernel_fwd)
+            fp, gp = fj.clone().requires_grad_(True), gj.clone().requires_grad_(True)
 
-        def chain_step():
-            fp.grad = gp.grad = Wp.grad = bp.grad = None
-            pkg.fused_joiner_loss(fp, gp, Wp, bp, lx, y, ly, 0, "mean", "tanh", total_rows=R, max_u=y.size(1),
-                                  one_kernel=True).backward()
+            def chain_step():
+                fp.grad = gp.grad = Wp.grad = bp.grad = None
+                pkg.fused_joiner_loss(fp, gp, Wp, bp, lx, y, ly, 0, "mean", "tanh", total_rows=R, max_u=y.size(1),
+                                      one_kernel=True).backward()
 
-        def two_kernel_step():
-            fp.grad = gp.grad = Wp.grad = bp.grad = None
-            hh = pkg.compact_join(fp, gp, lx, ly, "tanh", total_rows=R)
-            pkg.fused_joint_loss(hh, Wp, bp, lx, y, ly, 0, "mean", max_u=y.size(1)).backward()
+            def two_kernel_step():
+                fp.grad = gp.grad = Wp.grad = bp.grad = None
+                hh = pkg.compact_join(fp, gp, lx, ly, "tanh", total_rows=R)
+                pkg.fused_joint_loss(hh, Wp, bp, lx, y, ly, 0, "mean", max_u=y.size(1)).backward()
 
-        chain_ms = timed(chain_step)
-        two_ms = timed(two_kernel_step)
-        joiner_chain = {"what": "act(f[n,t] + g[n,u]) @ W^T + bias -> loss, tanh, f (N,T,H), g (N,U+1,H)",
-                        "forward_one_kernel_ms": round(chain_fwd, 4),
-                        "forward_one_kernel_keeping_rows_ms": round(chain_fwd_keep, 4),
-                        "forward_join_then_joint_ms": round(two_fwd, 4),
-                        "fwd_bwd_one_kernel_forward_ms": round(chain_ms, 4),
-                        "fwd_bwd_join_then_joint_ms": round(two_ms, 4)}
-        del fj, gj, fp, gp
+            chain_ms = timed(chain_step)
+            two_ms = timed(two_kernel_step)
+            joiner_chain = {"what": "act(f[n,t] + g[n,u]) @ W^T + bias -> loss, tanh, f (N,T,H), g (N,U+1,H)",
+                            "forward_one_kernel_ms": round(chain_fwd, 4),
+                            "forward_one_kernel_keeping_rows_ms": round(chain_fwd_keep, 4),
+                            "forward_join_then_joint_ms": round(two_fwd, 4),
+                            "fwd_bwd_one_kernel_forward_ms": round(chain_ms, 4),
+                            "fwd_bwd_join_then_joint_ms": round(two_ms, 4)}
+            del fj, gj, fp, gp
 
         torch.cuda.reset_peak_memory_stats()
         base_mem = torch.cuda.memory_allocated()

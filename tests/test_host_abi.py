@@ -329,3 +329,19 @@ def test_build_step_flags_a_scalar_select_on_a_stale_condition_code():
     via_mask = "\n".join(["\tv_cmp_eq_u32_e32 vcc, s20, v67", "\ts_and_b64 vcc, vcc, exec", "\ts_cselect_b32 s12, 0x7fffffff, s3"])
     assert [n for n, _ in stale_scc_reads(bad)] == [4]
     assert stale_scc_reads(good) == [] and stale_scc_reads(via_mask) == []
+
+
+def test_backward_blocks_of_the_fused_output_layer_are_equal_and_bounded():
+    """The default block of rows of fused_joint_loss's backward pass: the fewest blocks of at most
+    384 MiB of logit gradients (never fewer than 65536 rows), all of one size, a multiple of 256
+    rows, covering every row."""
+    from compactwarprnntloss_amd.joiner import _balanced_block
+    for R, V, size in [(311449, 1024, 2), (100, 1024, 2), (1_000_000, 1024, 2), (311449, 4096, 2), (400_000, 50_000, 2),
+                       (196_608, 1024, 2), (196_609, 1024, 2), (1, 8, 2)]:
+        block = _balanced_block(R, V, size)
+        limit = max(65536, (384 << 20) // (V * size))
+        blocks = -(-R // block)
+        assert block % 256 == 0 and block * blocks >= R
+        assert block <= (limit + 255) // 256 * 256
+        assert blocks == max(1, -(-R // limit))          # no more blocks than the limit asks for
+        assert block * blocks - R < 256 * blocks          # equal blocks: the last one is short by the rounding only
